@@ -1,0 +1,143 @@
+/* libm2_amd.so -- C ABI of the MI355X (gfx950) Monarch-Mixer forward kernels.
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream (as void*; pass 0 for the
+ * null stream) and enqueues work on that stream without synchronising.  The library allocates no
+ * device memory and keeps no device state: inputs, outputs and workspaces belong to the caller and
+ * must stay valid until the stream has run the enqueued kernels.  Return value: M2_OK (0) or a
+ * negative M2_ERR_* code, with a human-readable message available from m2_last_error() on the
+ * calling thread.  All matrices are dense and contiguous in the layouts stated per argument.
+ *
+ * The reference (HazyResearch/m2) binds its optional native kernels through the pybind11 module
+ * `flashmm` (csrc/flashmm/flash_mm.cpp:364-368: mm_block_fwd, hyena_filter_fwd,
+ * exp_mod_in_place_fwd) and otherwise runs the path as PyTorch ops.  The entry points below are
+ * what a binding for the same path would call; each cites the reference interface it stands in for.
+ */
+#ifndef M2_AMD_H_
+#define M2_AMD_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define M2_AMD_VERSION 100 /* major*10000 + minor*100 + patch */
+
+#define M2_OK 0
+#define M2_ERR_ARG (-1)         /* null pointer, non-positive size, bad enum */
+#define M2_ERR_UNSUPPORTED (-2) /* a size the kernels have no plan for */
+#define M2_ERR_LAUNCH (-3)      /* HIP reported an error at launch */
+
+#define M2_DTYPE_F32 0
+#define M2_DTYPE_BF16 1
+
+int m2_version(void);
+const char* m2_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Implicit long-filter generation (HyenaFilter.filter / filter_rev + ExponentialModulation).
+ * Stands in for: bert/src/mm/hyena_utils.py:201-217 (filter, filter_rev), :50-63 (Sin),
+ * :110-112 (modulation) and :231-236 (bidirectional padding/flip); native counterpart in the
+ * reference: flashmm.hyena_filter_fwd + exp_mod_in_place_fwd (csrc/flashmm/flash_mm.cpp:301-362).
+ * ------------------------------------------------------------------------------------------- */
+typedef struct m2_hyena_filter_params {
+  const float* z;      /* (L, emb_dim)  pos_emb.z[0, :L]                                  */
+  const float* t;      /* (L)           pos_emb.t[0, :L, 0]                               */
+  const float* freq;   /* (order)       Sin.freq (one tensor shared by all activations)   */
+  const float* deltas; /* (d)           modulation.deltas                                 */
+  const float* w0;     /* (order, emb_dim)  implicit_filter.0.weight                      */
+  const float* b0;     /* (order)           implicit_filter.0.bias                        */
+  const float* w1;     /* (order, order)    implicit_filter.2.weight                      */
+  const float* b1;     /* (order)                                                          */
+  const float* w2;     /* (order, order)    implicit_filter.4.weight                      */
+  const float* b2;     /* (order)                                                          */
+  const float* w3;     /* (d, order)        implicit_filter.6.weight (no bias)            */
+  const float* rw0;    /* same seven tensors of implicit_filter_rev; all NULL when the     */
+  const float* rb0;    /* filter is not bidirectional                                      */
+  const float* rw1;
+  const float* rb1;
+  const float* rw2;
+  const float* rb2;
+  const float* rw3;
+} m2_hyena_filter_params;
+
+/* Bytes of fp32 workspace m2_hyena_filter_fwd needs for `nfilters` filters of length L. */
+size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int order);
+
+/* taps[f] (d, 2L) fp32, f < nfilters:  taps[f][c][l]      = k_fwd[c][l]       for l < L
+ *                                      taps[f][c][L + l]  = k_rev[c][L-1-l]   (0 if not bidirectional)
+ * with k[c][l] = (W3 sin(f.(W2 sin(f.(W1 sin(f.(W0 z_l + b0)) + b1)) + b2)))[c] * (exp(-t_l |delta_c|) + shift),
+ * f = w_mod * freq.  `params` is a HOST array of nfilters structs holding DEVICE pointers.
+ * Supported: order == 128, 3 <= emb_dim <= 8, d % 64 == 0, L % 64 == 0. */
+int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order, int emb_dim,
+                        float w_mod, float shift, float* workspace, float* taps, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Long convolution: filter spectra and the fused mixer core.
+ * Stand in for: bert/src/mm/hyena_utils.py:16-42 (fftconv_ref), :219-248 (HyenaFilter.forward) and
+ * bert/src/mm/monarch_mixer_sequence_mixer.py:112-147 (short conv, gates, two long convs, add);
+ * native counterpart in the reference: flashmm.mm_block_fwd (csrc/flashmm/flash_mm.cpp:70-226).
+ * ------------------------------------------------------------------------------------------- */
+
+/* 1 if sequence length L is supported by the LDS-resident FFT (2L a power of two in [256, 16384]). */
+int m2_fftconv_supported_seqlen(int L);
+
+/* Bytes of the opaque spectrum buffer for d channels and sequence length L (both filters). */
+size_t m2_filter_spectrum_bytes(int d, int L);
+
+/* taps1, taps2: (d, 2L) fp32 bidirectional taps of filter_fn and filter_fn2 (taps2 may be NULL:
+ * treated as zero).  D1, D2: (d) fp32 skip weights (`filter_fn.bias`, `filter_fn2.bias`; either
+ * may be NULL = 0): the reference's "+ u * D" term (hyena_utils.py:35) equals adding D to tap 0,
+ * which is done here.  spec: m2_filter_spectrum_bytes(d, L) bytes; receives
+ * rfft(taps + D e0, 2L)/(2L) of both filters in the order m2_mixer_core_fwd reads them. */
+int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
+                           int d, int L, void* stream);
+
+/* y[c,b,:] = (fftconv(a; k1)[:L] + D1[c] a) * sc(x2) + fftconv(u; k2)[:L] + D2[c] u,
+ *            a = sc(v) * sc(x1),  sc = depthwise 3-tap causal conv + bias (cross-correlation,
+ *            out[t] = bias + w0 in[t-2] + w1 in[t-1] + w2 in[t]);  D1, D2 are already inside spec.
+ * xproj  (3d, B, L)  in_linear output, CHANNEL-MAJOR, channels [0,d)=x1, [d,2d)=x2, [2d,3d)=v; act_dtype
+ * u      (d, B, L)   fp32 layer input, channel-major; NULL when there is no residual long conv
+ * short_w (3d, 3), short_b (3d)  fp32
+ * spec   from m2_filter_spectrum_fwd with the same d and L
+ * y      (d, B, L)   act_dtype (M2_DTYPE_F32 or M2_DTYPE_BF16); FFT arithmetic is fp32 either way */
+int m2_mixer_core_fwd(const void* xproj, const float* u, const float* short_w, const float* short_b,
+                      const float* spec, void* y, int B, int L, int d, int act_dtype, void* stream);
+
+/* Plain long convolution y[c,b,:] = fftconv(x[c,b,:]; k1)[:L] + D1[c] x[c,b,:] with the first filter
+ * of `spec` (HyenaFilter.forward on its own, bert/src/mm/hyena_utils.py:219-248).
+ * x, y (d, B, L) channel-major, act_dtype. */
+int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, int L, int d, int act_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Block-diagonal ("Monarch") linear layers of the GLU MLP, bf16 MFMA with fp32 accumulation.
+ * Stand in for: bert/src/mm/blockdiag_multiply.py:49-60 (BlockdiagMultiply.forward, bf16 under
+ * autocast), bert/src/mm/structured_linear.py:65-69 (bias add) and bert/src/bert_layers.py:482-506
+ * (GLU, residual).  The reference has no native kernel for these (torch.bmm).
+ * ------------------------------------------------------------------------------------------- */
+
+/* out[m, j] = gelu_erf(h[m, j]) * h[m, I + j],  h = blockdiag_multiply(x, w),  j < I = intermediate.
+ * x (M, in_features) bf16 row-major; w (nblocks, 2I/nblocks, in_features/nblocks) bf16 (the
+ * `gated_layers.weight` tensor); out (M, I) bf16.  Needs nblocks even, (in/nblocks) % 16 == 0,
+ * (2I/nblocks) % 64 == 0. */
+int m2_blockdiag_glu_fwd(const void* x, const void* w, void* out, int M, int in_features, int intermediate,
+                         int nblocks, void* stream);
+
+/* out = blockdiag_multiply(x, w) (+ bias) (+ residual).
+ * x (M, in_features) bf16; w (nblocks, out/nblocks, in/nblocks) bf16; bias (out_features) fp32 or NULL;
+ * residual (M, out_features) bf16 or NULL; out (M, out_features) of out_dtype (M2_DTYPE_F32 / _BF16).
+ * Needs (in/nblocks) % 16 == 0, (out/nblocks) % 64 == 0. */
+int m2_blockdiag_linear_fwd(const void* x, const void* w, const float* bias, const void* residual, void* out, int M,
+                            int in_features, int out_features, int nblocks, int out_dtype, void* stream);
+
+/* LayerNorm over the last dimension of x (M, d) fp32 (torch.nn.LayerNorm semantics, biased variance,
+ * eps inside the root; bert/src/bert_layers.py:478-479,506 and :185-186,247).  Any of the three
+ * outputs may be NULL: out_f32 (M, d) fp32, out_bf16 (M, d) bf16, out_channel_major (d, M) fp32 (the
+ * layout m2_mixer_core_fwd reads its `u` in).  Needs d % 64 == 0, d <= 2048. */
+int m2_layernorm_fwd(const float* x, const float* gamma, const float* beta, float eps, float* out_f32, void* out_bf16,
+                     float* out_channel_major, int M, int d, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* M2_AMD_H_ */

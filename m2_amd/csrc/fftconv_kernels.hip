@@ -1,0 +1,654 @@
+// Fused Monarch-Mixer sequence-mixer core for gfx950, and the filter-spectrum kernel that feeds it.
+//
+// One (channel, batch) row of length L is convolved with two 2L-tap bidirectional filters by a
+// single complex FFT of length N = 2L held in LDS:
+//
+//   z[n] = a[n] + i*u[n]           a = shortconv(v) * shortconv(x1),  u = layer input   (n < L, 0 after)
+//   Z    = FFT_N(z)                in-place decimation in frequency, spectrum left digit-reversed
+//   A[k] = (Z[k] + conj Z[N-k])/2, B[k] = (Z[k] - conj Z[N-k])/(2i)      (spectra of a and of u)
+//   W[k] = A[k] K1[k] + i B[k] K2[k]
+//   w    = IFFT_N(W) (unscaled; K carries 1/N)  ->  Re w = a (*) k1,  Im w = u (*) k2
+//   y[n] = Re w[n] * shortconv(x2)[n] + Im w[n]                                        (n < L)
+//
+// The skip terms "+ D1 a" and "+ D2 u" of the reference are folded into tap 0 of the filters when
+// their spectra are built (k[0] += D), which is the same convolution.
+//
+// Replaces, for the reference's torch path, bert/src/mm/monarch_mixer_sequence_mixer.py:112-147
+// together with bert/src/mm/hyena_utils.py:16-42,231-236 (two fftconv_ref calls, the gating and the
+// residual add); the launch granularity corresponds to the reference's optional CUDA kernel
+// csrc/flashmm/mm_block_fwd_cuda.cu:173-647 but none of that code is used here.
+//
+// Thread mapping.  E = 16 complex points per thread, T = N/16 threads per row.  The FFT is
+// R1 x R2 (x R3) x 8.  Every pass but the last is "load R points at stride S, radix-R butterfly in
+// registers, twiddle, store in place".  The last forward pass and the first inverse pass are
+// radix-8 on contiguous groups of 8; thread w takes group g(w) AND the group g' that holds the
+// mirrored frequencies N-k, so the spectral multiply needs no exchange: it happens in registers
+// between the two radix-8 transforms.  The first forward pass reads straight from global memory
+// and the last inverse pass writes straight to global memory.
+//
+// The filter spectra are stored in exactly the order the multiply consumes them
+// ("native order": spec[channel][slot 0..7][w 0..T-1] as float4 = K1.re, K1.im, K2.re, K2.im for the
+// frequency that sits in slot `slot` of group g(w)); the spectrum kernel below produces that order
+// with the same FFT code, so the layout is private to this file.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fft_regs.h"
+#include "m2_internal.h"
+
+namespace m2 {
+
+// ------------------------------------------------------------------------------------------
+// plan
+// ------------------------------------------------------------------------------------------
+template <int LOGN_, int R1_, int R2_, int R3_>
+struct Plan {
+  static constexpr int LOGN = LOGN_, N = 1 << LOGN_, L = N / 2;
+  static constexpr int E = 16, RP = 8;
+  static constexpr int R1 = R1_, R2 = R2_, R3 = R3_;
+  static constexpr int T = N / E;            // threads per row
+  static constexpr int M = N / RP;           // groups of 8 in the last pass
+  static constexpr int S1 = N / R1, S2 = S1 / R2, S3 = S2 / R3;
+  static constexpr int RL = (R3 > 1) ? R3 : R2;   // radix of the least significant digit of a group index
+  static constexpr int WG = T < 256 ? 256 : T;    // threads per workgroup
+  static constexpr int RPW = WG / T;              // rows per workgroup
+  static constexpr int ROW_LDS = N + (N >> 4);    // padded complex slots per row
+  static_assert(R1 * R2 * R3 * RP == N, "radices must multiply to N");
+  static_assert(S3 == RP, "last stride");
+  static_assert(R1 * R2 >= E, "passes after the first must share twiddles inside a thread");
+};
+
+__device__ __forceinline__ int phys(int pos) { return pos + (pos >> 4); }
+
+// Padded offset of logical offset `o` relative to a base position whose low four bits, added to
+// (o mod 16), stay below 16.  True for every access below: strides are multiples of 16, or 8 with a
+// base offset below 8, or consecutive runs of 8 that start at a multiple of 8.
+constexpr int poff(int o) { return o + (o >> 4); }
+
+__device__ __forceinline__ cf lds_get(const float2* p, int off) {
+  float2 v = p[off];
+  return {v.x, v.y};
+}
+__device__ __forceinline__ void lds_put(float2* p, int off, cf v) { p[off] = make_float2(v.re, v.im); }
+
+// exp(-2*pi*i*m/n), n a power of two
+__device__ __forceinline__ cf unit_root(int m, int n) {
+  float s, c;
+  sincospif(2.0f * (float)m / (float)n, &s, &c);
+  return {c, -s};
+}
+
+// ------------------------------------------------------------------------------------------
+// generic passes on the row held in LDS
+// ------------------------------------------------------------------------------------------
+// forward: registers hold natural-order inputs of E/R butterflies; butterfly, twiddle, store.
+template <class P, int R, int S, bool ZERO_UPPER>
+__device__ __forceinline__ void fwd_compute_store(cf (&x)[16], int t, float2* row, const cf (&wbase)[16 / R]) {
+  constexpr int NB = 16 / R;
+  static_for<0, NB>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int q = t + P::T * i;
+    const int b = q / S, m = q % S;
+    if constexpr (ZERO_UPPER) dif_zero_upper<R, i * R, 16>(x);
+    else dif<R, i * R, 16>(x);
+    cf p[R];
+    powers<R>(wbase[(S > P::T) ? i : 0], p);
+    float2* pb = row + phys(b * (S * R) + m);
+    constexpr int bits = ilog2(R);
+    static_for<0, R>([&](auto kk) {
+      constexpr int k = decltype(kk)::value;
+      cf v = x[i * R + bitrev(k, bits)];
+      if constexpr (k > 0) v = cmul(v, p[k]);
+      lds_put(pb, poff(k * S), v);
+    });
+  });
+}
+
+template <class P, int R, int S>
+__device__ __forceinline__ void fwd_load(cf (&x)[16], int t, const float2* row) {
+  constexpr int NB = 16 / R;
+  static_for<0, NB>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int q = t + P::T * i;
+    const int b = q / S, m = q % S;
+    const float2* pb = row + phys(b * (S * R) + m);
+    static_for<0, R>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      x[i * R + j] = lds_get(pb, poff(j * S));
+    });
+  });
+}
+
+// inverse: load digit k into bit-reversed register, conj twiddle, inverse butterfly (natural out)
+template <class P, int R, int S, bool LOWER_ONLY>
+__device__ __forceinline__ void inv_load_compute(cf (&x)[16], int t, const float2* row, const cf (&wbase)[16 / R]) {
+  constexpr int NB = 16 / R;
+  static_for<0, NB>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int q = t + P::T * i;
+    const int b = q / S, m = q % S;
+    cf p[R];
+    powers<R>(wbase[(S > P::T) ? i : 0], p);
+    const float2* pb = row + phys(b * (S * R) + m);
+    constexpr int bits = ilog2(R);
+    static_for<0, R>([&](auto kk) {
+      constexpr int k = decltype(kk)::value;
+      cf v = lds_get(pb, poff(k * S));
+      if constexpr (k > 0) v = cmulc(v, p[k]);
+      x[i * R + bitrev(k, bits)] = v;
+    });
+    if constexpr (LOWER_ONLY) dit_lower_only<R, i * R, 16>(x);
+    else dit<R, i * R, 16>(x);
+  });
+}
+
+template <class P, int R, int S>
+__device__ __forceinline__ void inv_store(const cf (&x)[16], int t, float2* row) {
+  constexpr int NB = 16 / R;
+  static_for<0, NB>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int q = t + P::T * i;
+    const int b = q / S, m = q % S;
+    float2* pb = row + phys(b * (S * R) + m);
+    static_for<0, R>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      lds_put(pb, poff(j * S), x[i * R + j]);
+    });
+  });
+}
+
+// twiddle bases of one pass for thread t: exp(-2 pi i m / (S R)), one per butterfly when the
+// thread's butterflies have different offsets (first pass only), else a single shared one.
+template <class P, int R, int S>
+__device__ __forceinline__ void pass_bases(int t, cf (&w)[16 / R]) {
+  constexpr int NB = 16 / R;
+  static_for<0, NB>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    if constexpr (S > P::T || i == 0) {
+      const int q = t + P::T * i;
+      w[i] = unit_root(q % S, S * R);
+    } else {
+      w[i] = w[0];
+    }
+  });
+}
+
+// group taken by work item w in the paired radix-8 pass, and the group with the mirrored frequencies
+template <class P>
+__device__ __forceinline__ void paired_groups(int w, int& g, int& g2) {
+  constexpr int RL = P::RL, R1 = P::R1, R2 = P::R2, R3 = P::R3;
+  g = (w / (RL / 2)) * RL + (w % (RL / 2));
+  if (w == 0) {            // groups 0 (k_low = 0) and RL/2 (k_low = M/2) are both self-mirrored
+    g2 = RL / 2;
+    return;
+  }
+  int k1 = g / (R2 * R3), k2 = (g / R3) % R2, k3 = g % R3;
+  if (k1) {
+    k1 = R1 - k1; k2 = R2 - 1 - k2; k3 = R3 - 1 - k3;
+  } else if (k2) {
+    k2 = R2 - k2; k3 = R3 - 1 - k3;
+  } else {
+    k3 = R3 - k3;
+  }
+  g2 = (k1 * R2 + k2) * R3 + k3;
+}
+
+// ------------------------------------------------------------------------------------------
+// forward FFT up to (and including) the paired radix-8 pass.  On return x[0..8) holds group g
+// and x[8..16) holds group g2, both in bit-reversed register order.
+// ------------------------------------------------------------------------------------------
+template <class P, bool ZERO_UPPER>
+__device__ __forceinline__ void forward_to_pairs(cf (&x)[16], int t, float2* row, const cf (&wb1)[16 / P::R1],
+                                                 const cf (&wb2)[16 / P::R2], const cf (&wb3)[16 / P::R3],
+                                                 int g, int g2) {
+  fwd_compute_store<P, P::R1, P::S1, ZERO_UPPER>(x, t, row, wb1);
+  __syncthreads();
+  fwd_load<P, P::R2, P::S2>(x, t, row);
+  fwd_compute_store<P, P::R2, P::S2, false>(x, t, row, wb2);
+  __syncthreads();
+  if constexpr (P::R3 > 1) {
+    fwd_load<P, P::R3, P::S3>(x, t, row);
+    fwd_compute_store<P, P::R3, P::S3, false>(x, t, row, wb3);
+    __syncthreads();
+  }
+  {
+    const float2* pa = row + phys(g * 8);
+    const float2* pb = row + phys(g2 * 8);
+    static_for<0, 8>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      x[j] = lds_get(pa, j);
+      x[8 + j] = lds_get(pb, j);
+    });
+  }
+  dif<8, 0, 16>(x);
+  dif<8, 8, 16>(x);
+}
+
+// One spectral pair: za sits at frequency k, zb at N-k.  Returns W[k] in za and W[N-k] in zb.
+__device__ __forceinline__ void pair_multiply(cf& za, cf& zb, float4 K) {
+  cf A = {0.5f * (za.re + zb.re), 0.5f * (za.im - zb.im)};        // (Z[k] + conj Z[N-k]) / 2
+  cf Bq = {0.5f * (za.im + zb.im), 0.5f * (zb.re - za.re)};       // (Z[k] - conj Z[N-k]) / (2i)
+  cf Pp = cmul(A, cf{K.x, K.y});
+  cf Q = cmul(Bq, cf{K.z, K.w});
+  za = {Pp.re - Q.im, Pp.im + Q.re};                               // P + iQ
+  zb = {Pp.re + Q.im, Q.re - Pp.im};                               // conj(P) + i conj(Q)
+}
+
+// ------------------------------------------------------------------------------------------
+// K2: the fused mixer core
+// ------------------------------------------------------------------------------------------
+// 8 consecutive activations starting at element n0 (n0 % 8 == 0) plus the two before them, as fp32:
+// out[0], out[1] = in[n0-2], in[n0-1] (zero when n0 == 0), out[2..10) = in[n0 .. n0+8).
+__device__ __forceinline__ void load10(const float* p, int n0, float (&o)[10]) {
+  const float4 a = *reinterpret_cast<const float4*>(p + n0);
+  const float4 b = *reinterpret_cast<const float4*>(p + n0 + 4);
+  float2 h = make_float2(0.f, 0.f);
+  if (n0 > 0) h = *reinterpret_cast<const float2*>(p + n0 - 2);
+  o[0] = h.x; o[1] = h.y;
+  o[2] = a.x; o[3] = a.y; o[4] = a.z; o[5] = a.w;
+  o[6] = b.x; o[7] = b.y; o[8] = b.z; o[9] = b.w;
+}
+__device__ __forceinline__ void load10(const uint16_t* p, int n0, float (&o)[10]) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p + n0);
+  uint32_t h = 0;
+  if (n0 > 0) h = *reinterpret_cast<const uint32_t*>(p + n0 - 2);
+  o[0] = __uint_as_float(h << 16); o[1] = __uint_as_float(h & 0xffff0000u);
+  o[2] = __uint_as_float(a.x << 16); o[3] = __uint_as_float(a.x & 0xffff0000u);
+  o[4] = __uint_as_float(a.y << 16); o[5] = __uint_as_float(a.y & 0xffff0000u);
+  o[6] = __uint_as_float(a.z << 16); o[7] = __uint_as_float(a.z & 0xffff0000u);
+  o[8] = __uint_as_float(a.w << 16); o[9] = __uint_as_float(a.w & 0xffff0000u);
+}
+__device__ __forceinline__ void store8(float* p, int n0, const float (&v)[8]) {
+  *reinterpret_cast<float4*>(p + n0) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + n0 + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(uint16_t* p, int n0, const float (&v)[8]) {
+  uint4 o;
+  o.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+  o.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+  o.z = (uint32_t)f32_to_bf16(v[4]) | ((uint32_t)f32_to_bf16(v[5]) << 16);
+  o.w = (uint32_t)f32_to_bf16(v[6]) | ((uint32_t)f32_to_bf16(v[7]) << 16);
+  *reinterpret_cast<uint4*>(p + n0) = o;
+}
+
+// first forward pass when only positions [0, N/2) of the row are populated (upper half is zero)
+template <class P>
+__device__ __forceinline__ void fwd_load_lower(cf (&x)[16], int t, const float2* row) {
+  constexpr int R = P::R1, S = P::S1, NB = 16 / R;
+  static_for<0, NB>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const float2* pb = row + phys(t + P::T * i);
+    static_for<0, R / 2>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      x[i * R + j] = lds_get(pb, poff(j * S));
+    });
+  });
+}
+template <class P>
+__device__ __forceinline__ void inv_store_lower(const cf (&x)[16], int t, float2* row) {
+  constexpr int R = P::R1, S = P::S1, NB = 16 / R;
+  static_for<0, NB>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    float2* pb = row + phys(t + P::T * i);
+    static_for<0, R / 2>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      lds_put(pb, poff(j * S), x[i * R + j]);
+    });
+  });
+}
+
+template <class P, typename ACT>
+__global__ __launch_bounds__(P::WG) void mixer_core_kernel(
+    const ACT* __restrict__ xproj,      // (3d, B, L): x1 | x2 | v, channel-major
+    const float* __restrict__ uin,      // (d, B, L)   layer input, channel-major (may be null)
+    const float* __restrict__ sw,       // (3d, 3)     short-conv taps; null = plain convolution of a (d, B, L) input
+    const float* __restrict__ sb,       // (3d)        short-conv bias
+    const float4* __restrict__ spec,    // (d, 8, T)   native-order spectra
+    ACT* __restrict__ y,                // (d, B, L)
+    int B, int d) {
+  constexpr int L = P::L, T = P::T;
+  extern __shared__ float2 lds[];
+  const int tid = threadIdx.x;
+  const int rloc = tid / T, t = tid % T;
+  float2* row = lds + rloc * P::ROW_LDS;
+  const int nrows = d * B;
+  const int n0 = 8 * t;
+
+  cf wb1[16 / P::R1], wb2[16 / P::R2], wb3[16 / P::R3];
+  pass_bases<P, P::R1, P::S1>(t, wb1);
+  pass_bases<P, P::R2, P::S2>(t, wb2);
+  if constexpr (P::R3 > 1) pass_bases<P, P::R3, P::S3>(t, wb3);
+  int g, g2;
+  paired_groups<P>(t, g, g2);
+
+  for (int r0 = blockIdx.x * P::RPW; r0 < nrows; r0 += gridDim.x * P::RPW) {
+    const int r = r0 + rloc;
+    const bool valid = r < nrows;
+    const int rr = valid ? r : nrows - 1;
+    const int c = rr / B, b = rr % B;
+
+    // ---- prologue: 8 consecutive time steps per thread: short conv, gate, stage z = a + i u in LDS ----
+    float gate[8];
+    {
+      float in[10], a[8];
+      if (sw) {
+        const float* w = sw + (long)c * 3;
+        load10(xproj + ((long)(0 * d + c) * B + b) * L, n0, in);
+        {
+          const float w0 = w[0], w1 = w[1], w2 = w[2], bb = sb[c];
+          static_for<0, 8>([&](auto jj) {
+            constexpr int j = decltype(jj)::value;
+            a[j] = bb + w0 * in[j] + w1 * in[j + 1] + w2 * in[j + 2];
+          });
+        }
+        load10(xproj + ((long)(2 * d + c) * B + b) * L, n0, in);
+        {
+          const float w0 = w[6 * (long)d + 0], w1 = w[6 * (long)d + 1], w2 = w[6 * (long)d + 2], bb = sb[2 * d + c];
+          static_for<0, 8>([&](auto jj) {
+            constexpr int j = decltype(jj)::value;
+            a[j] *= bb + w0 * in[j] + w1 * in[j + 1] + w2 * in[j + 2];
+          });
+        }
+        load10(xproj + ((long)(1 * d + c) * B + b) * L, n0, in);
+        {
+          const float w0 = w[3 * (long)d + 0], w1 = w[3 * (long)d + 1], w2 = w[3 * (long)d + 2], bb = sb[d + c];
+          static_for<0, 8>([&](auto jj) {
+            constexpr int j = decltype(jj)::value;
+            gate[j] = bb + w0 * in[j] + w1 * in[j + 1] + w2 * in[j + 2];
+          });
+        }
+      } else {
+        // plain long convolution: xproj is a single (d, B, L) signal, no short conv, no gates
+        load10(xproj + ((long)c * B + b) * L, n0, in);
+        static_for<0, 8>([&](auto jj) {
+          constexpr int j = decltype(jj)::value;
+          a[j] = in[j + 2];
+          gate[j] = 1.f;
+        });
+      }
+      float4 u0 = make_float4(0.f, 0.f, 0.f, 0.f), u1 = u0;
+      if (uin) {
+        const float* pu = uin + ((long)c * B + b) * L + n0;
+        u0 = *reinterpret_cast<const float4*>(pu);
+        u1 = *reinterpret_cast<const float4*>(pu + 4);
+      }
+      float4* dst = reinterpret_cast<float4*>(row + phys(n0));     // 8 consecutive slots never straddle a pad
+      dst[0] = make_float4(a[0], u0.x, a[1], u0.y);
+      dst[1] = make_float4(a[2], u0.z, a[3], u0.w);
+      dst[2] = make_float4(a[4], u1.x, a[5], u1.y);
+      dst[3] = make_float4(a[6], u1.z, a[7], u1.w);
+    }
+    __syncthreads();
+
+    cf x[16];
+    fwd_load_lower<P>(x, t, row);
+    forward_to_pairs<P, true>(x, t, row, wb1, wb2, wb3, g, g2);
+
+    // ---- spectral multiply in registers ----
+    {
+      const float4* sp = spec + (long)c * 8 * T + t;
+      float4 K[8];
+      static_for<0, 8>([&](auto s) { K[decltype(s)::value] = sp[decltype(s)::value * T]; });
+      if (t != 0) {
+        static_for<0, 8>([&](auto jj) {
+          constexpr int j = decltype(jj)::value;
+          pair_multiply(x[bitrev(j, 3)], x[8 + bitrev(7 - j, 3)], K[j]);
+        });
+      } else {
+        // group 0: slots j <-> (8-j)%8 ; DC (j=0) and Nyquist (j=4) are self-paired and real-filtered
+        x[bitrev(0, 3)] = {x[bitrev(0, 3)].re * K[0].x, x[bitrev(0, 3)].im * K[0].z};
+        x[bitrev(4, 3)] = {x[bitrev(4, 3)].re * K[0].y, x[bitrev(4, 3)].im * K[0].w};
+        static_for<1, 4>([&](auto jj) {
+          constexpr int j = decltype(jj)::value;
+          pair_multiply(x[bitrev(j, 3)], x[bitrev(8 - j, 3)], K[j]);
+        });
+        // group RL/2 (k_low = M/2): slots j <-> 7-j inside the same group
+        static_for<0, 4>([&](auto jj) {
+          constexpr int j = decltype(jj)::value;
+          pair_multiply(x[8 + bitrev(j, 3)], x[8 + bitrev(7 - j, 3)], K[4 + j]);
+        });
+      }
+    }
+
+    // ---- inverse ----
+    dit<8, 0, 16>(x);
+    dit<8, 8, 16>(x);
+    {
+      float2* pa = row + phys(g * 8);
+      float2* pb = row + phys(g2 * 8);
+      static_for<0, 8>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        lds_put(pa, j, x[j]);
+        lds_put(pb, j, x[8 + j]);
+      });
+    }
+    __syncthreads();
+    if constexpr (P::R3 > 1) {
+      inv_load_compute<P, P::R3, P::S3, false>(x, t, row, wb3);
+      inv_store<P, P::R3, P::S3>(x, t, row);
+      __syncthreads();
+    }
+    inv_load_compute<P, P::R2, P::S2, false>(x, t, row, wb2);
+    inv_store<P, P::R2, P::S2>(x, t, row);
+    __syncthreads();
+    inv_load_compute<P, P::R1, P::S1, true>(x, t, row, wb1);
+    inv_store_lower<P>(x, t, row);      // only slots this thread has just read are overwritten
+    __syncthreads();
+
+    // ---- epilogue: 8 consecutive outputs per thread ----
+    {
+      const float4* src = reinterpret_cast<const float4*>(row + phys(n0));
+      const float4 o0 = src[0], o1 = src[1], o2 = src[2], o3 = src[3];
+      float out[8];
+      out[0] = o0.x * gate[0] + o0.y; out[1] = o0.z * gate[1] + o0.w;
+      out[2] = o1.x * gate[2] + o1.y; out[3] = o1.z * gate[3] + o1.w;
+      out[4] = o2.x * gate[4] + o2.y; out[5] = o2.z * gate[5] + o2.w;
+      out[6] = o3.x * gate[6] + o3.y; out[7] = o3.z * gate[7] + o3.w;
+      if (valid) store8(y + ((long)c * B + b) * L, n0, out);
+    }
+    __syncthreads();      // the next row's prologue overwrites what the epilogue has just read
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// K1c: filter taps -> native-order spectra (both filters of one mixer in one complex FFT)
+// ------------------------------------------------------------------------------------------
+template <class P>
+__global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
+    const float* __restrict__ taps1,    // (d, N) bidirectional taps of filter_fn
+    const float* __restrict__ taps2,    // (d, N) bidirectional taps of filter_fn2 (may be null)
+    const float* __restrict__ D1,       // (d) skip weight of filter_fn, added to tap 0 (may be null)
+    const float* __restrict__ D2,       // (d) skip weight of filter_fn2 (may be null)
+    float4* __restrict__ spec,          // (d, 8, T)
+    int d) {
+  constexpr int N = P::N, T = P::T;
+  extern __shared__ float2 lds[];
+  const int tid = threadIdx.x;
+  const int rloc = tid / T, t = tid % T;
+  float2* row = lds + rloc * P::ROW_LDS;
+  const int n0 = 16 * t;
+
+  cf wb1[16 / P::R1], wb2[16 / P::R2], wb3[16 / P::R3];
+  pass_bases<P, P::R1, P::S1>(t, wb1);
+  pass_bases<P, P::R2, P::S2>(t, wb2);
+  if constexpr (P::R3 > 1) pass_bases<P, P::R3, P::S3>(t, wb3);
+  int g, g2;
+  paired_groups<P>(t, g, g2);
+  const float scale = 0.5f / (float)N;       // the 1/2 of the even/odd split and the 1/N of the convolution
+
+  for (int r0 = blockIdx.x * P::RPW; r0 < d; r0 += gridDim.x * P::RPW) {
+    const int r = r0 + rloc;
+    const bool valid = r < d;
+    const int c = valid ? r : d - 1;
+    {   // 16 consecutive taps of each filter per thread -> z = k1 + i k2 staged in LDS
+      const float4* p1 = reinterpret_cast<const float4*>(taps1 + (long)c * N + n0);
+      float4* dst = reinterpret_cast<float4*>(row + phys(n0));
+      static_for<0, 4>([&](auto qq) {
+        constexpr int q = decltype(qq)::value;
+        float4 a = p1[q];
+        float4 bq = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (taps2) bq = reinterpret_cast<const float4*>(taps2 + (long)c * N + n0)[q];
+        if (q == 0 && t == 0) {          // the skip weight D is one more tap at lag 0
+          if (D1) a.x += D1[c];
+          if (D2) bq.x += D2[c];
+        }
+        dst[2 * q] = make_float4(a.x, bq.x, a.y, bq.y);
+        dst[2 * q + 1] = make_float4(a.z, bq.z, a.w, bq.w);
+      });
+    }
+    __syncthreads();
+    cf x[16];
+    fwd_load<P, P::R1, P::S1>(x, t, row);
+    forward_to_pairs<P, false>(x, t, row, wb1, wb2, wb3, g, g2);
+    __syncthreads();      // LDS is reused by the next row
+
+    float4 K[8];
+    auto split = [&](cf za, cf zb) -> float4 {
+      // K1 = (za + conj zb) * scale ; K2 = (za - conj zb) / i * scale
+      return make_float4(scale * (za.re + zb.re), scale * (za.im - zb.im), scale * (za.im + zb.im),
+                         scale * (zb.re - za.re));
+    };
+    if (t != 0) {
+      static_for<0, 8>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        K[j] = split(x[bitrev(j, 3)], x[8 + bitrev(7 - j, 3)]);
+      });
+    } else {
+      const cf z0 = x[bitrev(0, 3)], z4 = x[bitrev(4, 3)];
+      K[0] = make_float4(2.f * scale * z0.re, 2.f * scale * z4.re, 2.f * scale * z0.im, 2.f * scale * z4.im);
+      static_for<1, 4>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        K[j] = split(x[bitrev(j, 3)], x[bitrev(8 - j, 3)]);
+      });
+      static_for<0, 4>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        K[4 + j] = split(x[8 + bitrev(j, 3)], x[8 + bitrev(7 - j, 3)]);
+      });
+    }
+    if (valid) {
+      float4* sp = spec + (long)c * 8 * T + t;
+      static_for<0, 8>([&](auto s) { sp[decltype(s)::value * T] = K[decltype(s)::value]; });
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// host-side dispatch
+// ------------------------------------------------------------------------------------------
+template <class P, typename ACT>
+static int launch_mixer_core(const void* xproj, const float* u, const float* sw, const float* sb, const float* spec,
+                             void* y, int B, int d, hipStream_t stream) {
+  const size_t lds_bytes = (size_t)P::RPW * P::ROW_LDS * sizeof(float2);
+  auto kern = mixer_core_kernel<P, ACT>;
+  if (lds_bytes > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(mixer_core): %s", hipGetErrorString(e));
+  }
+  const int nrows = d * B;
+  const int wgs_needed = (nrows + P::RPW - 1) / P::RPW;
+  const int per_cu = (int)((160 * 1024) / lds_bytes) < 1 ? 1 : (int)((160 * 1024) / lds_bytes);
+  int grid = num_cus() * (per_cu > 8 ? 8 : per_cu);
+  if (grid > wgs_needed) grid = wgs_needed;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(P::WG), lds_bytes, stream, (const ACT*)xproj, u, sw, sb,
+                     (const float4*)spec, (ACT*)y, B, d);
+  return check_launch("mixer_core");
+}
+
+template <class P>
+static int launch_filter_spectrum(const float* taps1, const float* taps2, const float* D1, const float* D2,
+                                  float* spec, int d, hipStream_t stream) {
+  const size_t lds_bytes = (size_t)P::RPW * P::ROW_LDS * sizeof(float2);
+  auto kern = filter_spectrum_kernel<P>;
+  if (lds_bytes > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(filter_spectrum): %s", hipGetErrorString(e));
+  }
+  const int wgs_needed = (d + P::RPW - 1) / P::RPW;
+  int grid = num_cus() * 2;
+  if (grid > wgs_needed) grid = wgs_needed;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(P::WG), lds_bytes, stream, taps1, taps2, D1, D2, (float4*)spec, d);
+  return check_launch("filter_spectrum");
+}
+
+#define M2_FOR_EACH_PLAN(X) \
+  X(8, 4, 8, 1)             \
+  X(9, 8, 8, 1)             \
+  X(10, 16, 8, 1)           \
+  X(11, 16, 16, 1)          \
+  X(12, 8, 8, 8)            \
+  X(13, 16, 8, 8)           \
+  X(14, 16, 16, 8)
+
+}  // namespace m2
+
+using namespace m2;
+
+extern "C" int m2_fftconv_supported_seqlen(int L) {
+  int n = 2 * L;
+  return (n >= 256 && n <= 16384 && (n & (n - 1)) == 0) ? 1 : 0;
+}
+
+extern "C" size_t m2_filter_spectrum_bytes(int d, int L) {
+  return (size_t)d * (size_t)L * 16;        // d channels x 8 slots x (2L/16) work items x float4
+}
+
+extern "C" int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, const float* D1, const float* D2,
+                                      float* spec, int d, int L, void* stream) {
+  if (!taps1 || !spec) return set_error(M2_ERR_ARG, "m2_filter_spectrum_fwd: null pointer");
+  if (d <= 0) return set_error(M2_ERR_ARG, "m2_filter_spectrum_fwd: d must be positive, got %d", d);
+  if (!m2_fftconv_supported_seqlen(L))
+    return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: L=%d unsupported (need 2L a power of two in [256, 16384])", L);
+  const int logn = ilog2(2 * L);
+  switch (logn) {
+#define X(LOGN, R1, R2, R3) \
+  case LOGN:                \
+    return launch_filter_spectrum<Plan<LOGN, R1, R2, R3>>(taps1, taps2, D1, D2, spec, d, (hipStream_t)stream);
+    M2_FOR_EACH_PLAN(X)
+#undef X
+  }
+  return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: no plan for L=%d", L);
+}
+
+extern "C" int m2_mixer_core_fwd(const void* xproj, const float* u, const float* short_w, const float* short_b,
+                                 const float* spec, void* y, int B, int L, int d, int act_dtype, void* stream) {
+  if (!xproj || !short_w || !short_b || !spec || !y) return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: null pointer");
+  if (B <= 0 || d <= 0) return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: bad sizes B=%d d=%d", B, d);
+  if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
+    return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
+  if (!m2_fftconv_supported_seqlen(L))
+    return set_error(M2_ERR_UNSUPPORTED, "m2_mixer_core_fwd: L=%d unsupported (need 2L a power of two in [256, 16384])", L);
+  const int logn = ilog2(2 * L);
+  hipStream_t s = (hipStream_t)stream;
+  switch (logn) {
+#define X(LOGN, R1, R2, R3)                                                                                       \
+  case LOGN:                                                                                                      \
+    return act_dtype == M2_DTYPE_F32                                                                              \
+               ? launch_mixer_core<Plan<LOGN, R1, R2, R3>, float>(xproj, u, short_w, short_b, spec, y, B, d, s) \
+               : launch_mixer_core<Plan<LOGN, R1, R2, R3>, uint16_t>(xproj, u, short_w, short_b, spec, y, B, d, s);
+    M2_FOR_EACH_PLAN(X)
+#undef X
+  }
+  return set_error(M2_ERR_UNSUPPORTED, "m2_mixer_core_fwd: no plan for L=%d", L);
+}
+
+extern "C" int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, int L, int d, int act_dtype,
+                              void* stream) {
+  if (!x || !spec || !y) return set_error(M2_ERR_ARG, "m2_fftconv_fwd: null pointer");
+  if (B <= 0 || d <= 0) return set_error(M2_ERR_ARG, "m2_fftconv_fwd: bad sizes B=%d d=%d", B, d);
+  if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
+    return set_error(M2_ERR_ARG, "m2_fftconv_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
+  if (!m2_fftconv_supported_seqlen(L))
+    return set_error(M2_ERR_UNSUPPORTED, "m2_fftconv_fwd: L=%d unsupported (need 2L a power of two in [256, 16384])", L);
+  const int logn = ilog2(2 * L);
+  hipStream_t s = (hipStream_t)stream;
+  switch (logn) {
+#define X(LOGN, R1, R2, R3)                                                                                  \
+  case LOGN:                                                                                                 \
+    return act_dtype == M2_DTYPE_F32                                                                         \
+               ? launch_mixer_core<Plan<LOGN, R1, R2, R3>, float>(x, nullptr, nullptr, nullptr, spec, y, B, d, s) \
+               : launch_mixer_core<Plan<LOGN, R1, R2, R3>, uint16_t>(x, nullptr, nullptr, nullptr, spec, y, B, d, s);
+    M2_FOR_EACH_PLAN(X)
+#undef X
+  }
+  return set_error(M2_ERR_UNSUPPORTED, "m2_fftconv_fwd: no plan for L=%d", L);
+}

@@ -1,0 +1,31 @@
+// Helpers shared by the translation units of libm2_amd.so (not part of the public C ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/m2_amd.h"
+
+namespace m2 {
+
+// Records a printf-style message retrievable through m2_last_error() and returns `code`.
+int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+// hipGetLastError() after a launch -> 0 or M2_ERR_LAUNCH (message recorded).
+int check_launch(const char* what);
+// Compute units of the current device (cached per device).
+int num_cus();
+
+// round-to-nearest-even float -> bfloat16 bits (NaN stays NaN)
+__host__ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  union { float f; uint32_t u; } v;
+  v.f = f;
+  if ((v.u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((v.u >> 16) | 0x40u);
+  v.u += 0x7fffu + ((v.u >> 16) & 1u);
+  return (uint16_t)(v.u >> 16);
+}
+__host__ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
+  union { float f; uint32_t u; } v;
+  v.u = ((uint32_t)h) << 16;
+  return v.f;
+}
+
+}  // namespace m2

@@ -1,0 +1,212 @@
+"""M2-BERT encoder stack (Monarch-Mixer branch) over the HIP kernels, module and state-dict names as
+in the reference (bert/src/bert_layers.py:131-252 BertEmbeddings, :457-508 BertGatedLinearUnitMLP,
+:511-599 BertLayer, :602-813 BertEncoder, :880-1021 BertModel).
+
+`BertEncoder.forward` does not call its layers module by module: it runs one fused schedule per
+layer so that no activation is transposed or re-read in between:
+
+    h32 (M,d) f32, h16 (M,d) bf16, hT (d,M) f32   <- LayerNorm of the previous layer (three forms, one kernel)
+    xproj (3d,M) bf16 = W_in h16^T + b            library GEMM, channel-major output
+    spec              = filter spectra            K1 (hidden MLP, projection+decay) + spectrum FFT
+    y (d,M) bf16      = mixer core(xproj, hT)     K2
+    a (M,d) bf16      = y^T W_out^T + b           library GEMM
+    g (M,I) bf16      = GLU(blockdiag(a, Wg))     K3
+    s (M,d) f32       = blockdiag(g, Wo) + b + a  K3
+    LayerNorm(s)      -> next layer's three forms
+
+The individual modules keep working on their own (same call signatures as the reference) and give
+the same numbers; they just pay for the layout changes the fused schedule avoids.
+"""
+from __future__ import annotations
+
+from functools import partial
+from typing import List, Optional
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .blockdiag import BlockdiagLinear
+from .config import M2BertConfig
+from .mixer import MonarchMixerSequenceMixing
+
+
+class BertEmbeddings(nn.Module):
+    def __init__(self, config: M2BertConfig):
+        super().__init__()
+        self.word_embeddings = nn.Embedding(config.vocab_size, config.hidden_size, padding_idx=config.pad_token_id)
+        if config.use_positional_encodings:
+            self.position_embeddings = nn.Embedding(config.max_position_embeddings, config.hidden_size)
+        self.use_positional_encodings = config.use_positional_encodings
+        self.token_type_embeddings = nn.Embedding(config.type_vocab_size, config.hidden_size)
+        self.LayerNorm = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_eps)
+        self.dropout = nn.Dropout(config.hidden_dropout_prob)
+        if config.use_positional_encodings:
+            self.register_buffer("position_ids", torch.arange(config.max_position_embeddings).expand((1, -1)))
+        self.register_buffer("token_type_ids", torch.zeros(config.max_position_embeddings, dtype=torch.long),
+                             persistent=False)
+
+    def summed(self, input_ids=None, token_type_ids=None, position_ids=None, inputs_embeds=None,
+               past_key_values_length: int = 0) -> torch.Tensor:
+        """word + token-type (+ position) embeddings before the LayerNorm, (B, L, d) fp32."""
+        if (input_ids is not None) == (inputs_embeds is not None):
+            raise ValueError("Must specify either input_ids or input_embeds!")
+        shape = input_ids.size() if input_ids is not None else inputs_embeds.size()[:-1]
+        L = shape[1]
+        if inputs_embeds is None:
+            inputs_embeds = self.word_embeddings(input_ids)
+        if token_type_ids is None:
+            tt = self.token_type_embeddings.weight[0]            # all-zero type ids
+            e = inputs_embeds + tt
+        else:
+            e = inputs_embeds + self.token_type_embeddings(token_type_ids)
+        if self.use_positional_encodings:
+            if position_ids is None:
+                position_ids = self.position_ids[:, past_key_values_length:L + past_key_values_length]
+            e = e + self.position_embeddings(position_ids)
+        return e
+
+    def forward(self, input_ids=None, token_type_ids=None, position_ids=None, inputs_embeds=None,
+                past_key_values_length: int = 0) -> torch.Tensor:
+        if self.training and self.dropout.p > 0:
+            raise NotImplementedError("m2_amd is a forward/inference path: call .eval() first")
+        e = self.summed(input_ids, token_type_ids, position_ids, inputs_embeds, past_key_values_length).float()
+        B, L, d = e.shape
+        o32, _, _ = ops.layernorm(e.reshape(B * L, d).contiguous(), self.LayerNorm.weight.detach().float(),
+                                  self.LayerNorm.bias.detach().float(), self.LayerNorm.eps)
+        return o32.view(B, L, d)
+
+
+class BertGatedLinearUnitMLP(nn.Module):
+    def __init__(self, config: M2BertConfig):
+        super().__init__()
+        if not config.use_monarch_mlp:
+            raise NotImplementedError("only the Monarch (block-diagonal) GLU MLP is built")
+        self.config = config
+        self.is_padded = config.monarch_mixer_sequence_mixing
+        linear_cls = partial(BlockdiagLinear, nblocks=config.monarch_mlp_nblocks)
+        self.gated_layers = linear_cls(config.hidden_size, config.intermediate_size * 2, bias=False)
+        self.act = nn.GELU(approximate="none")
+        self.wo = linear_cls(config.intermediate_size, config.hidden_size)
+        self.dropout = nn.Dropout(config.hidden_dropout_prob)
+        self.layernorm = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_eps)
+
+    def presum(self, a16: torch.Tensor) -> torch.Tensor:
+        """a16 (M, d) bf16 -> wo(glu(a16)) + bias + a16, (M, d) fp32 (the LayerNorm input)."""
+        g = ops.blockdiag_glu(a16, self.gated_layers.weight_bf16())
+        return ops.blockdiag_linear(g, self.wo.weight_bf16(), self.wo.bias.detach().float().contiguous(), a16,
+                                    out_dtype=torch.float32)
+
+    def ln_params(self):
+        return self.layernorm.weight.detach().float(), self.layernorm.bias.detach().float(), self.layernorm.eps
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        if self.training and self.dropout.p > 0:
+            raise NotImplementedError("m2_amd is a forward/inference path: call .eval() first")
+        shape = hidden_states.shape
+        a16 = hidden_states.reshape(-1, shape[-1]).to(torch.bfloat16).contiguous()
+        s = self.presum(a16)
+        gamma, beta, eps = self.ln_params()
+        o32, _, _ = ops.layernorm(s, gamma, beta, eps)
+        return o32.view(shape)
+
+
+class BertLayer(nn.Module):
+    def __init__(self, config: M2BertConfig):
+        super().__init__()
+        if not config.monarch_mixer_sequence_mixing or not config.use_glu_mlp:
+            raise NotImplementedError("only the Monarch-Mixer branch with the GLU MLP is built")
+        self.monarch_mixer_sequence_mixing = True
+        self.attention = MonarchMixerSequenceMixing(
+            config.hidden_size, l_max=config.long_conv_l_max, hyena_kernel_lr=config.long_conv_kernel_learning_rate,
+            bidirectional=config.bidirectional, hyena_lr_pos_emb=config.hyena_lr_pos_emb, hyena_w=config.hyena_w,
+            hyena_w_mod=config.hyena_w_mod, hyena_wd=config.hyena_wd, hyena_emb_dim=config.hyena_emb_dim,
+            hyena_filter_dropout=config.hyena_filter_dropout, hyena_filter_order=config.hyena_filter_order,
+            residual_long_conv=config.residual_long_conv, hyena_training_additions=config.hyena_training_additions)
+        self.mlp = BertGatedLinearUnitMLP(config)
+
+    def forward(self, hidden_states, cu_seqlens=None, seqlen=None, subset_idx=None, indices=None, attn_mask=None,
+                bias=None) -> torch.Tensor:
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            a, _ = self.attention(hidden_states)
+        return self.mlp(a)
+
+    def fused(self, h16: torch.Tensor, hT: Optional[torch.Tensor], B: int, L: int, want_f32: bool):
+        """One layer of the fused schedule.  h16 (M,d) bf16, hT (d,M) f32 -> (f32 | None, bf16, (d,M) f32)."""
+        at = self.attention
+        d = at.d_model
+        w_in = at._cast("in_w", at.in_linear.weight, torch.bfloat16)
+        b_in = at._cast("in_b", at.in_linear.bias, torch.bfloat16)
+        w_out = at._cast("out_w", at.out_linear.weight, torch.bfloat16)
+        b_out = at._cast("out_b", at.out_linear.bias, torch.bfloat16)
+        xproj = torch.addmm(b_in.unsqueeze(1), w_in, h16.t())                        # (3d, M)
+        y = at.core(xproj.view(3 * d, B, L), hT.view(d, B, L) if at.residual_long_conv else None, B, L)
+        a16 = torch.addmm(b_out, y.view(d, B * L).t(), w_out.t())                    # (M, d)
+        s = self.mlp.presum(a16)
+        gamma, beta, eps = self.mlp.ln_params()
+        return ops.layernorm(s, gamma, beta, eps, want_f32=want_f32, want_bf16=True, want_channel_major=True)
+
+
+class BertEncoder(nn.Module):
+    def __init__(self, config: M2BertConfig):
+        super().__init__()
+        self.layer = nn.ModuleList([BertLayer(config) for _ in range(config.num_hidden_layers)])
+        self.monarch_mixer_sequence_mixing = config.monarch_mixer_sequence_mixing
+        self.num_attention_heads = config.num_attention_heads
+
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                output_all_encoded_layers: Optional[bool] = True, subset_mask: Optional[torch.Tensor] = None,
+                position_encodings: Optional[torch.Tensor] = None) -> List[torch.Tensor]:
+        """hidden_states (B, L, d) -> list of (B, L, d) fp32.  `attention_mask` is accepted and, as in the
+        reference's Monarch-Mixer branch (bert/src/bert_layers.py:577,721-726), never used."""
+        if not hidden_states.is_cuda:
+            raise RuntimeError("BertEncoder (m2_amd) runs on the GPU only")
+        if position_encodings is not None:
+            raise NotImplementedError("position_encodings added after every layer is not built")
+        B, L, d = hidden_states.shape
+        M = B * L
+        h32 = hidden_states.reshape(M, d).float().contiguous()
+        with torch.autocast("cuda", enabled=False):
+            h16 = h32.to(torch.bfloat16)
+            hT = h32.t().contiguous()
+            outs = []
+            n = len(self.layer)
+            for i, layer in enumerate(self.layer):
+                want = output_all_encoded_layers or i == n - 1
+                o32, h16, hT = layer.fused(h16, hT, B, L, want_f32=want)
+                if output_all_encoded_layers:
+                    outs.append(o32.view(B, L, d))
+            last = o32.view(B, L, d)
+        if subset_mask is not None:
+            last = last[subset_mask]
+            if output_all_encoded_layers:
+                outs[-1] = last
+        if not output_all_encoded_layers:
+            outs.append(last)
+        return outs
+
+
+class BertModel(nn.Module):
+    """Embeddings + encoder (no pooler: the heads are outside the accelerated path)."""
+
+    def __init__(self, config: M2BertConfig, add_pooling_layer: bool = False):
+        super().__init__()
+        if add_pooling_layer:
+            raise NotImplementedError("pooler / heads are not part of this path")
+        self.config = config
+        self.embeddings = BertEmbeddings(config)
+        self.encoder = BertEncoder(config)
+        self.pooler = None
+
+    def get_input_embeddings(self):
+        return self.embeddings.word_embeddings
+
+    def forward(self, input_ids: torch.Tensor, token_type_ids: Optional[torch.Tensor] = None,
+                attention_mask: Optional[torch.Tensor] = None, position_ids: Optional[torch.Tensor] = None,
+                output_all_encoded_layers: Optional[bool] = False, masked_tokens_mask: Optional[torch.Tensor] = None,
+                **kwargs):
+        if masked_tokens_mask is not None:
+            raise NotImplementedError("masked_tokens_mask subsetting belongs to the MLM head, which is not built")
+        emb = self.embeddings(input_ids, token_type_ids, position_ids)
+        enc = self.encoder(emb, attention_mask, output_all_encoded_layers=output_all_encoded_layers)
+        return (enc if output_all_encoded_layers else enc[-1]), None

@@ -1,0 +1,107 @@
+"""MonarchMixerSequenceMixing with the reference's constructor and state dict, computed by the fused
+HIP mixer core (bert/src/mm/monarch_mixer_sequence_mixer.py:12-154).
+
+Data flow of `forward(u)`, u (B, L, d):
+
+    xproj (3d, B*L) = in_linear.weight @ u^T + bias       one library GEMM, written CHANNEL-major
+    spec            = spectra of the two bidirectional implicit filters (skip weights folded in)
+    y (d, B*L)      = m2_mixer_core_fwd(xproj, u^T, short_filter, spec)
+    out (B*L, d)    = y^T @ out_linear.weight^T + bias     one library GEMM
+
+so the three `transpose` passes of the reference disappear into GEMM operand orientation.  With fp32
+input outside autocast everything is fp32; with bf16 input or under CUDA autocast the projections
+and the stored activations are bf16 while the FFT convolution stays fp32.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .hyena import HyenaFilter
+
+
+class MonarchMixerSequenceMixing(nn.Module):
+    def __init__(self, d_model, l_max=128, dropout=0.0, hyena_kernel_lr=None, bidirectional=False,
+                 hyena_lr_pos_emb=1e-5, hyena_w=10, hyena_w_mod=1, hyena_wd=0.1, hyena_emb_dim=3,
+                 hyena_filter_dropout=0.0, hyena_filter_order=16, residual_long_conv=False,
+                 hyena_training_additions=False):
+        super().__init__()
+        if hyena_training_additions:
+            raise NotImplementedError("hyena_training_additions=True (extra LayerNorm/dropout) is not built")
+        self.d_model = d_model
+        self.l_max = l_max
+        self.kernel_lr = hyena_kernel_lr
+        self.channels = 1
+        self.bidirectional = bidirectional
+        self.residual_long_conv = residual_long_conv
+        self.NUM_PROJECTIONS = 3
+        self.hyena_training_additions = hyena_training_additions
+
+        def make_filter():
+            return HyenaFilter(self.d_model, order=hyena_filter_order, seq_len=self.l_max, dropout=hyena_filter_dropout,
+                               bidirectional=self.bidirectional, lr=hyena_kernel_lr, lr_pos_emb=hyena_lr_pos_emb,
+                               w=hyena_w, w_mod=hyena_w_mod, wd=hyena_wd, emb_dim=hyena_emb_dim)
+
+        self.filter_fn = make_filter()
+        if self.residual_long_conv:
+            self.filter_fn2 = make_filter()
+        self.in_linear = nn.Linear(d_model, 3 * d_model)
+        self.out_linear = nn.Linear(d_model, d_model)
+        total_width = self.d_model * self.NUM_PROJECTIONS
+        self.short_filter = nn.Conv1d(in_channels=total_width, out_channels=total_width, kernel_size=3,
+                                      groups=total_width, padding=2)
+        self._cast_cache = {}
+
+    # -- helpers -----------------------------------------------------------------------------
+    def _cast(self, name: str, p: torch.Tensor, dtype) -> torch.Tensor:
+        """Cached cast of a parameter (re-done when the parameter changes)."""
+        key = (name, dtype)
+        tag = (p.data_ptr(), p._version, p.device)
+        hit = self._cast_cache.get(key)
+        if hit is None or hit[0] != tag:
+            hit = (tag, p.detach().to(dtype).contiguous())
+            self._cast_cache[key] = hit
+        return hit[1]
+
+    def filter_spectrum(self, L: int) -> torch.Tensor:
+        """Spectra of filter_fn (and filter_fn2) for sequence length L, generated from the weights."""
+        fns = [self.filter_fn] + ([self.filter_fn2] if self.residual_long_conv else [])
+        f0 = self.filter_fn
+        taps = ops.hyena_filter_taps([f.kernel_params("both") for f in fns], L, self.d_model, f0.order, f0.emb_dim,
+                                     w_mod=float(f0.w_mod), shift=float(f0.modulation.shift))
+        D1 = self.filter_fn.bias.detach().float().contiguous()
+        D2 = self.filter_fn2.bias.detach().float().contiguous() if self.residual_long_conv else None
+        return ops.filter_spectrum(taps[0], taps[1] if self.residual_long_conv else None, D1, D2)
+
+    def core(self, xproj: torch.Tensor, u_cm: Optional[torch.Tensor], B: int, L: int,
+             spec: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Channel-major core: xproj (3d, B, L), u_cm (d, B, L) fp32 -> y (d, B, L)."""
+        if spec is None:
+            spec = self.filter_spectrum(L)
+        sw = self._cast("short_w", self.short_filter.weight, torch.float32).view(3 * self.d_model, 3)
+        sb = self._cast("short_b", self.short_filter.bias, torch.float32)
+        return ops.mixer_core(xproj, u_cm, sw, sb, spec, B, L, self.d_model)
+
+    # -- reference API -----------------------------------------------------------------------
+    def forward(self, u, **kwargs):
+        if not u.is_cuda:
+            raise RuntimeError("MonarchMixerSequenceMixing (m2_amd) runs on the GPU only")
+        B, L, d = u.shape
+        if d != self.d_model:
+            raise ValueError(f"expected last dim {self.d_model}, got {d}")
+        low = u.dtype == torch.bfloat16 or torch.is_autocast_enabled()
+        act = torch.bfloat16 if low else torch.float32
+        u2 = u.reshape(B * L, d)
+        w_in = self._cast("in_w", self.in_linear.weight, act)
+        b_in = self._cast("in_b", self.in_linear.bias, act)
+        w_out = self._cast("out_w", self.out_linear.weight, act)
+        b_out = self._cast("out_b", self.out_linear.bias, act)
+        with torch.autocast("cuda", enabled=False):
+            xproj = torch.addmm(b_in.unsqueeze(1), w_in, u2.to(act).t())              # (3d, B*L)
+            u_cm = u2.float().t().contiguous() if self.residual_long_conv else None      # (d, B*L)
+            y = self.core(xproj.view(3 * d, B, L), None if u_cm is None else u_cm.view(d, B, L), B, L)
+            out = torch.addmm(b_out, y.view(d, B * L).t(), w_out.t())                   # (B*L, d)
+        return out.view(B, L, d), None

@@ -1,0 +1,194 @@
+"""Tensor-level wrappers over the C ABI of libm2_amd.so.
+
+PyTorch is used here for device memory and streams only: each function validates shapes, dtypes,
+devices and contiguity in Python (the library re-checks sizes), allocates the output with
+`torch.empty`, and enqueues the HIP kernels on torch's current stream.  CPU tensors are rejected:
+there is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import HyenaFilterParams, M2_DTYPE_BF16, M2_DTYPE_F32, check, lib
+
+Tensor = torch.Tensor
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require(t: Tensor, name: str, dtype=None, shape=None) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name}: must live on the GPU (m2_amd has no CPU path); got device {t.device}")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name}: expected dtype {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: must be contiguous")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
+
+
+def _ptr(t: Optional[Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _act_code(dtype) -> int:
+    if dtype == torch.float32:
+        return M2_DTYPE_F32
+    if dtype == torch.bfloat16:
+        return M2_DTYPE_BF16
+    raise TypeError(f"activation dtype must be float32 or bfloat16, got {dtype}")
+
+
+def fftconv_supported(L: int) -> bool:
+    return bool(lib.m2_fftconv_supported_seqlen(int(L)))
+
+
+# ------------------------------------------------------------------------------------------------
+def hyena_filter_taps(filters: Sequence[dict], L: int, d: int, order: int, emb_dim: int, w_mod: float = 1.0,
+                      shift: float = 0.0) -> Tensor:
+    """Bidirectional taps (nfilters, d, 2L) fp32 of `filters`.
+
+    Each entry is a dict with fp32 GPU tensors: z (>=L, emb), t (>=L), freq (order), deltas (d),
+    `fwd` = [w0, b0, w1, b1, w2, b2, w3] and optionally `rev` = the same seven of the reverse MLP.
+    """
+    nf = len(filters)
+    arr = (HyenaFilterParams * nf)()
+    keep = []
+    for i, f in enumerate(filters):
+        z = f["z"].reshape(-1, emb_dim)[:L].contiguous()
+        t = f["t"].reshape(-1)[:L].contiguous()
+        freq = f["freq"].reshape(-1).contiguous()
+        deltas = f["deltas"].reshape(-1).contiguous()
+        _require(z, "z", torch.float32, (L, emb_dim))
+        _require(t, "t", torch.float32, (L,))
+        _require(freq, "freq", torch.float32, (order,))
+        _require(deltas, "deltas", torch.float32, (d,))
+        keep += [z, t, freq, deltas]
+        arr[i].z, arr[i].t, arr[i].freq, arr[i].deltas = z.data_ptr(), t.data_ptr(), freq.data_ptr(), deltas.data_ptr()
+        shapes = [(order, emb_dim), (order,), (order, order), (order,), (order, order), (order,), (d, order)]
+        for key, names in (("fwd", ("w0", "b0", "w1", "b1", "w2", "b2", "w3")),
+                           ("rev", ("rw0", "rb0", "rw1", "rb1", "rw2", "rb2", "rw3"))):
+            ws = f.get(key)
+            if ws is None:
+                if key == "fwd":
+                    raise ValueError("filter without forward MLP")
+                continue
+            for w, n, s in zip(ws, names, shapes):
+                w = w.contiguous()
+                _require(w, f"{key}.{n}", torch.float32, s)
+                keep.append(w)
+                setattr(arr[i], n, w.data_ptr())
+    dev = keep[0].device
+    ws_bytes = lib.m2_hyena_filter_workspace_bytes(nf, L, order)
+    workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
+    taps = torch.empty(nf, d, 2 * L, dtype=torch.float32, device=dev)
+    check(lib.m2_hyena_filter_fwd(arr, nf, L, d, order, emb_dim, float(w_mod), float(shift), _ptr(workspace),
+                                  _ptr(taps), _stream()))
+    return taps
+
+
+def filter_spectrum(taps1: Tensor, taps2: Optional[Tensor], D1: Optional[Tensor], D2: Optional[Tensor]) -> Tensor:
+    """Opaque spectrum buffer for `mixer_core` from (d, 2L) taps of one or two filters."""
+    d, n = taps1.shape
+    L = n // 2
+    _require(taps1, "taps1", torch.float32, (d, 2 * L))
+    if taps2 is not None:
+        _require(taps2, "taps2", torch.float32, (d, 2 * L))
+    for nm, D in (("D1", D1), ("D2", D2)):
+        if D is not None:
+            _require(D, nm, torch.float32, (d,))
+    spec = torch.empty(lib.m2_filter_spectrum_bytes(d, L) // 4, dtype=torch.float32, device=taps1.device)
+    check(lib.m2_filter_spectrum_fwd(_ptr(taps1), _ptr(taps2), _ptr(D1), _ptr(D2), _ptr(spec), d, L, _stream()))
+    return spec
+
+
+def mixer_core(xproj: Tensor, u: Optional[Tensor], short_w: Tensor, short_b: Tensor, spec: Tensor, B: int, L: int,
+               d: int, out: Optional[Tensor] = None) -> Tensor:
+    """y (d, B, L) from the channel-major in-projection (3d, B, L) and layer input (d, B, L)."""
+    _require(xproj, "xproj", None, (3 * d, B, L))
+    code = _act_code(xproj.dtype)
+    if u is not None:
+        _require(u, "u", torch.float32, (d, B, L))
+    _require(short_w, "short_w", torch.float32, (3 * d, 3))
+    _require(short_b, "short_b", torch.float32, (3 * d,))
+    _require(spec, "spec", torch.float32, (lib.m2_filter_spectrum_bytes(d, L) // 4,))
+    if out is None:
+        out = torch.empty(d, B, L, dtype=xproj.dtype, device=xproj.device)
+    else:
+        _require(out, "out", xproj.dtype, (d, B, L))
+    check(lib.m2_mixer_core_fwd(_ptr(xproj), _ptr(u), _ptr(short_w), _ptr(short_b), _ptr(spec), _ptr(out), B, L, d,
+                                code, _stream()))
+    return out
+
+
+def fftconv(x: Tensor, spec: Tensor, B: int, L: int, d: int) -> Tensor:
+    """Plain long convolution of x (d, B, L) with the first filter held in `spec` (skip term included)."""
+    _require(x, "x", None, (d, B, L))
+    code = _act_code(x.dtype)
+    _require(spec, "spec", torch.float32, (lib.m2_filter_spectrum_bytes(d, L) // 4,))
+    out = torch.empty_like(x)
+    check(lib.m2_fftconv_fwd(_ptr(x), _ptr(spec), _ptr(out), B, L, d, code, _stream()))
+    return out
+
+
+def blockdiag_glu(x: Tensor, w: Tensor, out: Optional[Tensor] = None) -> Tensor:
+    """gelu_erf(h[:, :I]) * h[:, I:] with h = blockdiag_multiply(x, w); x (M, in) bf16, w (nb, 2I/nb, in/nb) bf16."""
+    M, in_f = x.shape
+    nb, q, p = w.shape
+    _require(x, "x", torch.bfloat16)
+    _require(w, "w", torch.bfloat16)
+    if nb * p != in_f:
+        raise ValueError(f"x has {in_f} features, weight expects {nb}*{p}")
+    I = nb * q // 2
+    if out is None:
+        out = torch.empty(M, I, dtype=torch.bfloat16, device=x.device)
+    else:
+        _require(out, "out", torch.bfloat16, (M, I))
+    check(lib.m2_blockdiag_glu_fwd(_ptr(x), _ptr(w), _ptr(out), M, in_f, I, nb, _stream()))
+    return out
+
+
+def blockdiag_linear(x: Tensor, w: Tensor, bias: Optional[Tensor] = None, residual: Optional[Tensor] = None,
+                     out_dtype=torch.bfloat16, out: Optional[Tensor] = None) -> Tensor:
+    """blockdiag_multiply(x, w) (+ bias) (+ residual); x (M, in) bf16, w (nb, out/nb, in/nb) bf16."""
+    M, in_f = x.shape
+    nb, q, p = w.shape
+    _require(x, "x", torch.bfloat16)
+    _require(w, "w", torch.bfloat16)
+    if nb * p != in_f:
+        raise ValueError(f"x has {in_f} features, weight expects {nb}*{p}")
+    out_f = nb * q
+    if bias is not None:
+        _require(bias, "bias", torch.float32, (out_f,))
+    if residual is not None:
+        _require(residual, "residual", torch.bfloat16, (M, out_f))
+    if out is None:
+        out = torch.empty(M, out_f, dtype=out_dtype, device=x.device)
+    else:
+        _require(out, "out", out_dtype, (M, out_f))
+    check(lib.m2_blockdiag_linear_fwd(_ptr(x), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out), M, in_f, out_f, nb,
+                                      _act_code(out_dtype), _stream()))
+    return out
+
+
+def layernorm(x: Tensor, gamma: Tensor, beta: Tensor, eps: float, want_f32: bool = True, want_bf16: bool = False,
+              want_channel_major: bool = False):
+    """LayerNorm over the last dim of x (M, d) fp32 -> (f32 (M,d) | None, bf16 (M,d) | None, f32 (d,M) | None)."""
+    M, d = x.shape
+    _require(x, "x", torch.float32)
+    _require(gamma, "gamma", torch.float32, (d,))
+    _require(beta, "beta", torch.float32, (d,))
+    o32 = torch.empty(M, d, dtype=torch.float32, device=x.device) if want_f32 else None
+    o16 = torch.empty(M, d, dtype=torch.bfloat16, device=x.device) if want_bf16 else None
+    ot = torch.empty(d, M, dtype=torch.float32, device=x.device) if want_channel_major else None
+    check(lib.m2_layernorm_fwd(_ptr(x), _ptr(gamma), _ptr(beta), float(eps), _ptr(o32), _ptr(o16), _ptr(ot), M, d,
+                               _stream()))
+    return o32, o16, ot

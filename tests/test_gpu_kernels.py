@@ -1,0 +1,177 @@
+"""GPU parity of each C-ABI entry point against the CPU oracle (same seeded inputs).
+
+Tolerances: fp32 long-convolution path 1e-4 relative (max-abs error over max-abs reference);
+bf16 GEMM paths 2e-2 relative.
+"""
+import math
+
+import pytest
+import torch
+
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL_F32 = 1e-4
+TOL_BF16 = 2e-2
+
+
+def _cfg(L, d=128, layers=1, I=None):
+    import m2_amd
+    cfg = m2_amd.M2BertConfig(hidden_size=d, intermediate_size=I or 4 * d, num_hidden_layers=layers).with_seq_len(L)
+    return cfg
+
+
+@pytest.mark.parametrize("L", [128, 256, 1024])
+@pytest.mark.parametrize("std", [0.02, 0.3])
+def test_hyena_filter_taps(gpu, L, std):
+    """K1 vs oracle.hyena_filter_taps; std=0.3 drives the sin arguments far outside [-pi, pi]."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    cfg = _cfg(L, d=192)
+    sd = m2_amd.seeded_state_dict(cfg, 7, std=std, what="mixer")
+    mix = m2_amd.MonarchMixerSequenceMixing(cfg.hidden_size, l_max=L, bidirectional=True, hyena_emb_dim=5,
+                                            hyena_filter_order=128, residual_long_conv=True, hyena_w=10)
+    mix.load_state_dict(sd)
+    mix = mix.to(gpu)
+    sd64 = O.cast_state_dict(sd, torch.float64)
+    for fn, name in ((mix.filter_fn, "filter_fn."), (mix.filter_fn2, "filter_fn2.")):
+        taps = fn.bidirectional_taps(L).cpu()
+        kf = O.hyena_filter_taps(sd64, name, L, rev=False)[0].T
+        kr = O.hyena_filter_taps(sd64, name, L, rev=True)[0].T
+        ref = O.bidirectional_kernel(kf, kr, L)
+        e, _ = rel_err(taps, ref)
+        assert e < 2e-5, (name, e)
+        # reference API shapes
+        h = fn.filter(L)
+        assert h.shape == (1, L, cfg.hidden_size)
+        assert rel_err(h.cpu(), kf.T[None])[0] < 2e-5
+        hr = fn.filter_rev(L)
+        assert rel_err(hr.cpu(), kr.T[None])[0] < 2e-5
+
+
+@pytest.mark.parametrize("L", [128, 256, 512, 1024, 2048, 4096, 8192])
+@pytest.mark.parametrize("act", ["f32", "bf16"])
+def test_mixer_core(gpu, L, act):
+    """K1c + K2 vs the oracle's short conv / gating / two fftconvs, every FFT plan."""
+    import m2_amd
+    from m2_amd import ops
+    from oracle import m2_oracle as O
+    d, B = 64, 3
+    g = torch.Generator().manual_seed(100 + L)
+    dt = torch.float32 if act == "f32" else torch.bfloat16
+    xproj = torch.randn(3 * d, B, L, generator=g).to(dt)
+    u = torch.randn(d, B, L, generator=g)
+    sw = torch.randn(3 * d, 3, generator=g) * 0.5
+    sb = torch.randn(3 * d, generator=g) * 0.1
+    t = torch.linspace(0, 1, 2 * L)
+    taps = [torch.randn(d, 2 * L, generator=g) * torch.exp(-4 * torch.minimum(t, 1 - t)) for _ in range(2)]
+    D = [torch.randn(d, generator=g) for _ in range(2)]
+    spec = ops.filter_spectrum(taps[0].to(gpu), taps[1].to(gpu), D[0].to(gpu), D[1].to(gpu))
+    y = ops.mixer_core(xproj.to(gpu), u.to(gpu), sw.to(gpu), sb.to(gpu), spec, B, L, d)
+    # oracle in float64 on the same (possibly bf16-rounded) inputs
+    x64 = xproj.double().permute(1, 0, 2)                      # (B, 3d, L)
+    uc = O.short_conv(x64, sw.double().view(3 * d, 1, 3), sb.double())
+    x1, x2, v = uc.split(d, dim=1)
+    y1 = O.fftconv(v * x1, taps[0].double(), D[0].double()[None, :, None])
+    y2 = O.fftconv(u.double().permute(1, 0, 2), taps[1].double(), D[1].double()[None, :, None])
+    ref = (y1 * x2 + y2).permute(1, 0, 2)
+    e, e2 = rel_err(y.float(), ref)
+    tol = TOL_F32 if act == "f32" else 6e-3        # bf16 output rounding is 2^-9
+    assert e < tol, (L, act, e, e2)
+
+
+def test_plain_fftconv_module_api(gpu):
+    """HyenaFilter.forward(x, L, k_fwd, k_rev, bias) keeps the reference call shape."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    L, d, B = 256, 64, 2
+    g = torch.Generator().manual_seed(5)
+    fn = m2_amd.HyenaFilter(d, emb_dim=5, order=128, seq_len=L, bidirectional=True, w=10).to(gpu)
+    x = torch.randn(B, d, L, generator=g)
+    kf = torch.randn(d, L, generator=g) * 0.1
+    kr = torch.randn(d, L, generator=g) * 0.1
+    bias = torch.randn(d, generator=g)
+    y = fn(x.to(gpu), L, k_fwd=kf.to(gpu), k_rev=kr.to(gpu), bias=bias.to(gpu)[None, :, None])
+    ref = O.hyena_filter_forward(x.double(), L, kf.double(), kr.double(), bias.double()[None, :, None])
+    assert rel_err(y, ref)[0] < TOL_F32
+
+
+@pytest.mark.parametrize("M,d,I", [(256, 768, 3072), (200, 256, 512), (4096, 1536, 6144)])
+def test_blockdiag_glu_and_linear(gpu, M, d, I):
+    """K3 vs oracle.blockdiag_* on bf16-rounded operands (fp64 reference)."""
+    from m2_amd import ops
+    from oracle import m2_oracle as O
+    nb = 4
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(M, d, generator=g).bfloat16()
+    wg = (torch.randn(nb, 2 * I // nb, d // nb, generator=g) * 0.05).bfloat16()
+    wo = (torch.randn(nb, d // nb, I // nb, generator=g) * 0.05).bfloat16()
+    bias = torch.randn(d, generator=g)
+    got = ops.blockdiag_glu(x.to(gpu), wg.to(gpu))
+    h = O.blockdiag_multiply(x.double(), wg.double())
+    ref = torch.nn.functional.gelu(h[:, :I]) * h[:, I:]
+    assert rel_err(got.float(), ref)[0] < TOL_BF16
+    a = ref.bfloat16()
+    got2 = ops.blockdiag_linear(a.to(gpu), wo.to(gpu), bias.to(gpu), x.to(gpu), out_dtype=torch.float32)
+    ref2 = O.blockdiag_multiply(a.double(), wo.double()) + bias.double() + x.double()
+    assert rel_err(got2, ref2)[0] < 1e-3        # fp32 accumulate of exact bf16 products
+    got3 = ops.blockdiag_linear(a.to(gpu), wo.to(gpu), None, None, out_dtype=torch.bfloat16)
+    assert rel_err(got3.float(), O.blockdiag_multiply(a.double(), wo.double()))[0] < TOL_BF16
+
+
+@pytest.mark.parametrize("M,d", [(300, 768), (64, 1536), (1000, 128)])
+def test_layernorm_three_outputs(gpu, M, d):
+    from m2_amd import ops
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(M, d, generator=g) * 3 + 1
+    gamma = torch.randn(d, generator=g)
+    beta = torch.randn(d, generator=g)
+    o32, o16, ot = ops.layernorm(x.to(gpu), gamma.to(gpu), beta.to(gpu), 1e-12, True, True, True)
+    ref = torch.nn.functional.layer_norm(x.double(), (d,), gamma.double(), beta.double(), 1e-12)
+    assert rel_err(o32, ref)[0] < 1e-5
+    assert rel_err(ot.T, ref)[0] < 1e-5
+    assert rel_err(o16.float(), ref)[0] < 6e-3
+
+
+def test_config1_mixer_fp32(gpu):
+    """BASELINE config 1: one MonarchMixerSequenceMixing layer, fp32, B=16 L=128 d=768, tol 1e-4."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    cfg = m2_amd.m2_bert_80m(128)
+    sd = m2_amd.seeded_state_dict(cfg, 1234, what="mixer")
+    mix = m2_amd.MonarchMixerSequenceMixing(768, l_max=128, bidirectional=True, hyena_emb_dim=5, hyena_filter_order=128,
+                                            residual_long_conv=True, hyena_w=10, hyena_w_mod=1)
+    mix.load_state_dict(sd)
+    mix = mix.to(gpu).eval()
+    u = torch.randn(16, 128, 768, generator=torch.Generator().manual_seed(1234))
+    y, none = mix(u.to(gpu))
+    assert none is None and y.dtype == torch.float32 and y.shape == u.shape
+    ref = O.mixer_forward(sd, "", u)
+    e, e2 = rel_err(y, ref)
+    assert e < TOL_F32 and e2 < TOL_F32, (e, e2)
+
+
+@pytest.mark.parametrize("L,B,layers", [(128, 4, 2), (1024, 2, 2)])
+def test_encoder_small(gpu, L, B, layers):
+    """Fused encoder schedule and the module-by-module path agree with the oracle (bf16 tolerance)."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    cfg = m2_amd.m2_bert_80m(L)
+    cfg.num_hidden_layers = layers
+    sd = m2_amd.seeded_state_dict(cfg, 99)
+    model = m2_amd.BertModel(cfg)
+    model.load_state_dict(sd)
+    model = model.to(gpu).eval()
+    ids = torch.randint(0, cfg.vocab_size, (B, L), generator=torch.Generator().manual_seed(5))
+    mask = torch.ones(B, L, dtype=torch.long)
+    out, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
+    ref = O.model_forward(sd, ids, mask, cfg)
+    e, e2 = rel_err(out, ref)
+    assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
+    # layer-by-layer module path
+    x = model.embeddings(ids.to(gpu))
+    for layer in model.encoder.layer:
+        x = layer(x)
+    e, e2 = rel_err(x, ref)
+    assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
