@@ -41,13 +41,17 @@ def test_hyena_filter_taps(gpu, L, std):
         kr = O.hyena_filter_taps(sd64, name, L, rev=True)[0].T
         ref = O.bidirectional_kernel(kf, kr, L)
         e, _ = rel_err(taps, ref)
-        assert e < 2e-5, (name, e)
+        # yardstick: how far the fp32 CPU oracle itself is from fp64 (sin(10 x) amplifies rounding)
+        ref32 = O.bidirectional_kernel(O.hyena_filter_taps(sd, name, L, rev=False)[0].T,
+                                       O.hyena_filter_taps(sd, name, L, rev=True)[0].T, L)
+        e32, _ = rel_err(ref32, ref)
+        assert e < max(2e-5, 4 * e32), (name, e, e32)
         # reference API shapes
         h = fn.filter(L)
         assert h.shape == (1, L, cfg.hidden_size)
-        assert rel_err(h.cpu(), kf.T[None])[0] < 2e-5
+        assert rel_err(h.cpu(), kf.T[None])[0] < max(2e-5, 4 * e32)
         hr = fn.filter_rev(L)
-        assert rel_err(hr.cpu(), kr.T[None])[0] < 2e-5
+        assert rel_err(hr.cpu(), kr.T[None])[0] < max(2e-5, 4 * e32)
 
 
 @pytest.mark.parametrize("L", [128, 256, 512, 1024, 2048, 4096, 8192])
