@@ -1,0 +1,202 @@
+#!/usr/bin/env python3
+"""Throughput of the M2-BERT-80M encoder forward on one MI355X, sequences per second.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c2|c5|c1] [--no-cpu-baseline]
+
+A step is one forward of embeddings + 12 Monarch-Mixer layers over one synthetic batch that is
+already resident in HBM (token ids on the GPU; filters are regenerated from the weights in every
+forward, as the reference does).  The default workload is the one the headline metric is quoted on:
+L = 8192, batch 4 (BASELINE config index 2).  One JSON line is printed:
+
+  value / ms_per_step   whole forward, wall clock bracketed by torch.cuda.synchronize()
+  roofline              the fused mixer-core kernel: algorithmic bytes per launch divided by its average
+                        duration, measured with HIP events around every launch inside the timed steps
+  cpu_baseline          the CPU oracle (plain PyTorch fp32 restatement of the reference path) timed on
+                        this host's cores on the same inputs and weights
+
+Only one GPU is used; --gpus N with N > 1 exits with a message.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def workload(name: str):
+    import m2_amd
+    if name == "c3":
+        cfg, B, pad = m2_amd.m2_bert_80m(8192), 4, True
+        label = "M2-BERT-80M encoder fwd, L=8192, B=4, padded lengths U[4096,8192] (config 2)"
+        idx = 2
+    elif name == "c2":
+        cfg, B, pad = m2_amd.m2_bert_80m(128), 32, False
+        label = "M2-BERT-80M encoder fwd, L=128, B=32 (config 1)"
+        idx = 1
+    elif name == "c5":
+        cfg, B, pad = m2_amd.m2_bert_large(128, 24), 64, False
+        label = "M2-BERT large 24x1536 encoder fwd, L=128, B=64 (config 4)"
+        idx = 4
+    else:
+        raise SystemExit(f"unknown config {name}")
+    gen = torch.Generator().manual_seed(1234 + idx)
+    L = cfg.max_position_embeddings
+    ids = torch.randint(0, cfg.vocab_size, (B, L), generator=gen)
+    mask = torch.ones(B, L, dtype=torch.long)
+    if pad:
+        lens = torch.randint(L // 2, L + 1, (B,), generator=gen)
+        for b in range(B):
+            ids[b, lens[b]:] = cfg.pad_token_id
+            mask[b, lens[b]:] = 0
+    return cfg, B, L, ids, mask, label, idx
+
+
+def mixer_core_bytes(B: int, L: int, d: int, act_bytes: int = 2) -> int:
+    """Algorithmic HBM bytes of one mixer-core launch: read x1,x2,v (act), read the fp32 layer input,
+    write y (act), read the four L-tap fp32 filters (= the two spectra) once."""
+    M = B * L
+    return M * 3 * d * act_bytes + M * d * 4 + M * d * act_bytes + 4 * d * L * 4
+
+
+class KernelTimer:
+    """HIP-event pairs around selected launches on torch's current stream (where the kernels run)."""
+
+    def __init__(self):
+        self.pairs = {}
+
+    def wrap(self, module, fn_name: str, tag: str):
+        orig = getattr(module, fn_name)
+
+        def timed(*a, **k):
+            s = torch.cuda.Event(enable_timing=True)
+            e = torch.cuda.Event(enable_timing=True)
+            s.record()
+            out = orig(*a, **k)
+            e.record()
+            self.pairs.setdefault(tag, []).append((s, e))
+            return out
+
+        setattr(module, fn_name, timed)
+        return orig
+
+    def reset(self):
+        self.pairs = {}
+
+    def mean_ms(self, tag: str) -> float:
+        p = self.pairs.get(tag, [])
+        return sum(s.elapsed_time(e) for s, e in p) / max(1, len(p))
+
+    def count(self, tag: str) -> int:
+        return len(self.pairs.get(tag, []))
+
+
+def cpu_baseline(sd, cfg, ids, mask, B):
+    from oracle import m2_oracle as O
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    with torch.no_grad():
+        x = O.embeddings_forward(sd, "embeddings.", ids, cfg)
+        O.layer_forward(sd, "encoder.layer.0.", x, cfg)            # warm-up: one layer
+        t0 = time.perf_counter()
+        ref = O.model_forward(sd, ids, mask, cfg)
+        dt = time.perf_counter() - t0
+    return ref, {"value": B / dt, "unit": "seq/s", "cores": torch.get_num_threads(), "kind": "port",
+                 "sample": f"one full forward (embeddings + {cfg.num_hidden_layers} layers) of the same batch, "
+                           f"fp32 torch.fft/einsum oracle, {dt:.2f} s after a one-layer warm-up"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c3")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+
+    import m2_amd
+    from m2_amd import ops
+
+    cfg, B, L, ids, mask, label, idx = workload(args.config)
+    d = cfg.hidden_size
+    sd = m2_amd.seeded_state_dict(cfg, 1234 + idx)
+    dev = torch.device("cuda:0")
+    model = m2_amd.BertModel(cfg)
+    model.load_state_dict(sd)
+    model = model.to(dev).eval()
+    ids_g, mask_g = ids.to(dev), mask.to(dev)
+
+    timer = KernelTimer()
+    timer.wrap(ops, "mixer_core", "mixer_core")
+    timer.wrap(ops, "hyena_filter_taps", "filter_taps")
+    timer.wrap(ops, "filter_spectrum", "filter_spectrum")
+    timer.wrap(ops, "blockdiag_glu", "blockdiag_glu")
+    timer.wrap(ops, "blockdiag_linear", "blockdiag_linear")
+    timer.wrap(ops, "layernorm", "layernorm")
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            out, _ = model(ids_g, attention_mask=mask_g)
+        torch.cuda.synchronize()
+        timer.reset()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out, _ = model(ids_g, attention_mask=mask_g)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    ms = dt / args.steps * 1e3
+    value = B / (dt / args.steps)
+
+    t_core = timer.mean_ms("mixer_core")
+    t_filt = timer.mean_ms("filter_taps") + timer.mean_ms("filter_spectrum")
+    nbytes = mixer_core_bytes(B, L, d, 2)
+    achieved = nbytes / (t_core * 1e-3) / 1e9
+    I = cfg.intermediate_size
+    M = B * L
+    glu_flops = 2 * M * d * 2 * I / cfg.monarch_mlp_nblocks
+    wo_flops = 2 * M * I * d / cfg.monarch_mlp_nblocks
+    t_glu, t_wo = timer.mean_ms("blockdiag_glu"), timer.mean_ms("blockdiag_linear")
+
+    result = {
+        "metric": "seq/s M2-BERT-80M fwd at L=8192; FFT-conv HBM GB/s & % of peak" if args.config == "c3"
+        else f"seq/s encoder fwd ({args.config})",
+        "value": value, "unit": "seq/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 GEMM / f32 FFT", "data": "synthetic token ids, seeded N(0,0.02) weights",
+        "config": {"workload": label, "batch": B, "seq_len": L, "d_model": d, "layers": cfg.num_hidden_layers,
+                   "filters": "regenerated from weights every forward"},
+        "roofline": {"kernel": "mixer_core_kernel (short conv + gates + two FFT long convs + add)",
+                     "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "bytes_per_launch": nbytes, "ms_per_launch": t_core, "launches_timed": timer.count("mixer_core"),
+                     "achieved_incl_filter_generation": nbytes / ((t_core + t_filt) * 1e-3) / 1e9,
+                     "filter_generation_ms_per_layer": t_filt},
+        "kernels_ms_per_layer": {"mixer_core": t_core, "filter_taps": timer.mean_ms("filter_taps"),
+                                 "filter_spectrum": timer.mean_ms("filter_spectrum"), "blockdiag_glu": t_glu,
+                                 "blockdiag_linear": t_wo, "layernorm": timer.mean_ms("layernorm")},
+        "blockdiag_mfma": {"glu_tflops": glu_flops / (t_glu * 1e-3) / 1e12, "wo_tflops": wo_flops / (t_wo * 1e-3) / 1e12,
+                           "peak_tflops": 2500.0,
+                           "frac": (glu_flops + wo_flops) / ((t_glu + t_wo) * 1e-3) / 1e12 / 2500.0},
+    }
+    if not args.no_cpu_baseline:
+        ref, cb = cpu_baseline(sd, cfg, ids, mask, B)
+        result["cpu_baseline"] = cb
+        o = out.float().cpu().double()
+        r = ref.double()
+        result["parity_vs_cpu_oracle"] = {"max_rel": ((o - r).abs().max() / r.abs().max()).item(),
+                                          "l2_rel": ((o - r).norm() / r.norm()).item(), "tolerance": 2e-2}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
