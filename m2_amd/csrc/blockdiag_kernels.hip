@@ -11,28 +11,52 @@
 //
 // MFMA: v_mfma_f32_32x32x16_bf16.  Lane (i = lane % 32, h = lane / 32) supplies A[i][8h .. 8h+7] and
 // B[8h .. 8h+7][i]; both operands are K-contiguous in memory (x row-major, w[k] is (q, p)), so every
-// operand register is one 16-byte load.  Accumulator element v of a lane is row 8 (v/4) + 4 h + v%4,
+// operand register is one 16-byte LDS read.  Accumulator element v of a lane is row 8 (v/4) + 4 h + v%4,
 // column i.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fft_regs.h"
 #include "m2_internal.h"
 
 namespace m2 {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ bf16x8 ld8(const uint16_t* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
 
-__device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+// x * Phi(x) with Phi through erfc(z) ~= P(t) exp(-z^2), t = 1/(1 + p z), z = |x|/sqrt2 (Abramowitz-Stegun
+// 7.1.26, |error in erfc| <= 1.5e-7).  The negative branch uses erfc directly, so the tail keeps its
+// relative accuracy; the result is rounded to bf16 by the caller.
+__device__ __forceinline__ float gelu_erf(float x) {
+  const float z = fabsf(x) * 0.70710678118654752440f;
+  const float t = __frcp_rn(fmaf(0.3275911f, z, 1.0f));
+  float poly = fmaf(1.061405429f, t, -1.453152027f);
+  poly = fmaf(poly, t, 1.421413741f);
+  poly = fmaf(poly, t, -0.284496736f);
+  poly = fmaf(poly, t, 0.254829592f);
+  const float erfc_z = poly * t * __expf(-z * z);
+  return x >= 0.f ? x * fmaf(-0.5f, erfc_z, 1.0f) : 0.5f * x * erfc_z;
+}
 
-// Workgroup = 4 waves as 2 (rows) x 2 (cols); wave tile 64 rows x 32 cols; workgroup tile 128 x 64.
-// grid (ceil(M / 128), ncol_tiles) where ncol_tiles counts 64-wide tiles over the OUTPUT columns
-// (I for GLU, out_features otherwise).  Requires q % 64 == 0 (GLU: (q) % 64 == 0 too), p % 16 == 0.
-template <bool GLU, typename OUT>
+// ---------------------------------------------------------------------------------------------
+// LDS-tiled GEMM core.  Workgroup = 4 waves laid out WR x WC; wave tile 64 x 64 (2 x 2 MFMA tiles);
+// workgroup tile BM = 64 WR rows by BN = 64 WC output columns.  K advances in chunks of 64: global
+// memory -> registers -> LDS (rows padded to 144 bytes so that the 16-byte operand reads of 32
+// consecutive rows fall in distinct banks), double buffered, one barrier per chunk.  The finished
+// tile goes back through LDS so that every global store is a full contiguous row segment.
+//
+// GLU: the chunk sequence runs the gate GEMM (block kb) and then the value GEMM (block kb + nb/2) of
+// the same output columns; gelu(gate) is parked in registers as packed bf16 between the two.
+// ---------------------------------------------------------------------------------------------
+constexpr int kBK = 64;
+constexpr int kLdsRow = kBK + 8;          // bf16 elements per padded LDS row (144 bytes)
+
+template <int WR, int WC, bool GLU, typename OUT, int NSTAGE>
 __global__ __launch_bounds__(256) void blockdiag_kernel(
     const uint16_t* __restrict__ x,      // (M, nb p) bf16
     const uint16_t* __restrict__ w,      // (nb, q, p) bf16
@@ -40,106 +64,248 @@ __global__ __launch_bounds__(256) void blockdiag_kernel(
     const uint16_t* __restrict__ resid,  // (M, nb q) bf16 or null    [GLU: unused]
     OUT* __restrict__ out,               // GLU: (M, nb q / 2) ; else (M, nb q)
     int M, int nb, int p, int q) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i32 = lane & 31, half = lane >> 5;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.x * 128 + wm * 64;
-  const int n0 = blockIdx.y * 64 + wn * 32;          // output column of this wave's tile
+  constexpr int BM = 64 * WR, BN = 64 * WC;
+  constexpr int A_CH = BM * (kBK / 8) / 256, B_CH = BN * (kBK / 8) / 256;      // 16-byte chunks per thread
+  constexpr int STAGE = (BM + BN) * kLdsRow;                                   // bf16 elements per stage
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
+  const int wr = wave / WC, wc = wave % WC;
+  // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  XCD e takes the row
+  // tiles e, e+8, ... and walks all column tiles of one row tile back to back, so the x rows and the
+  // weights of the tiles in flight on an XCD stay in that XCD's L2.
+  int tile_m, tile_n;
+  {
+    const int ntm = (M + BM - 1) / BM, ntn = (GLU ? nb * q / 2 : nb * q) / BN;
+    const int id = blockIdx.x, e = id & 7, l = id >> 3;
+    const int full = (ntm / 8) * 8;                   // row tiles covered by the XCD-striped part
+    if (id < full * ntn) {
+      tile_m = (l / ntn) * 8 + e;
+      tile_n = l % ntn;
+    } else {                                          // remainder rows: plain order
+      const int rid = id - full * ntn;
+      tile_m = full + rid / ntn;
+      tile_n = rid % ntn;
+    }
+  }
+  const int m0 = tile_m * BM;
+  const int n0 = tile_n * BN;                         // first output column of the tile
   const int in_f = nb * p;
-  const int blk = n0 / q, jj = n0 % q;               // block and column inside the block (gate block for GLU)
+  const int blk = n0 / q, jj = n0 % q;                // weight block and first row inside it (gate block for GLU)
   const int out_cols = GLU ? nb * q / 2 : nb * q;
+  const int kchunks = p / kBK;
+  const int nchunks = GLU ? 2 * kchunks : kchunks;
 
-  // rows beyond M are clamped for loads and masked at the store
-  int rowA[2];
-  for (int a = 0; a < 2; ++a) {
-    int r = m0 + 32 * a + i32;
-    rowA[a] = r < M ? r : M - 1;
-  }
-  const uint16_t* xg = x + (long)blk * p + 8 * half;
-  const uint16_t* wg = w + ((long)blk * q + jj + i32) * p + 8 * half;
-  const uint16_t* xv = GLU ? x + (long)(blk + nb / 2) * p + 8 * half : nullptr;
-  const uint16_t* wv = GLU ? w + ((long)(blk + nb / 2) * q + jj + i32) * p + 8 * half : nullptr;
+  // per-thread source rows of the 16-byte chunks it moves (fixed for the whole kernel)
+  const uint16_t* pa[A_CH];
+  const uint16_t* pb[B_CH];
+  int la[A_CH], lb[B_CH];
+  static_for<0, A_CH>([&](auto jj_) {
+    constexpr int j = decltype(jj_)::value;
+    const int id = tid + 256 * j, r = id >> 3, kc = id & 7;
+    int row = m0 + r;
+    row = row < M ? row : M - 1;
+    pa[j] = x + (long)row * in_f + (long)blk * p + kc * 8;
+    la[j] = r * kLdsRow + kc * 8;
+  });
+  static_for<0, B_CH>([&](auto jj_) {
+    constexpr int j = decltype(jj_)::value;
+    const int id = tid + 256 * j, r = id >> 3, kc = id & 7;
+    pb[j] = w + ((long)blk * q + jj + r) * p + kc * 8;
+    lb[j] = (BM + r) * kLdsRow + kc * 8;
+  });
+  const long a_phase = (long)(nb / 2) * p;            // value block = gate block + nb/2
+  const long b_phase = (long)(nb / 2) * q * p;
 
-  floatx16 accg[2], accv[2];
-  for (int a = 0; a < 2; ++a)
-    for (int v = 0; v < 16; ++v) { accg[a][v] = 0.f; accv[a][v] = 0.f; }
+  u32x4 ra[A_CH], rb[B_CH];
+  auto gload = [&](int c) __attribute__((always_inline)) {
+    const int phase = GLU ? c / kchunks : 0;
+    const long ao = phase * a_phase + (c % kchunks) * kBK;
+    const long bo = phase * b_phase + (c % kchunks) * kBK;
+    static_for<0, A_CH>([&](auto jj_) { ra[decltype(jj_)::value] = *reinterpret_cast<const u32x4*>(pa[decltype(jj_)::value] + ao); });
+    static_for<0, B_CH>([&](auto jj_) { rb[decltype(jj_)::value] = *reinterpret_cast<const u32x4*>(pb[decltype(jj_)::value] + bo); });
+  };
+  auto sstore = [&](int stage) __attribute__((always_inline)) {
+    uint16_t* st = smem + stage * STAGE;
+    static_for<0, A_CH>([&](auto jj_) { *reinterpret_cast<u32x4*>(st + la[decltype(jj_)::value]) = ra[decltype(jj_)::value]; });
+    static_for<0, B_CH>([&](auto jj_) { *reinterpret_cast<u32x4*>(st + lb[decltype(jj_)::value]) = rb[decltype(jj_)::value]; });
+  };
 
-  for (int k = 0; k < p; k += 16) {
-    const bf16x8 bg = ld8(wg + k);
-    bf16x8 ag[2];
-    for (int a = 0; a < 2; ++a) ag[a] = ld8(xg + (long)rowA[a] * in_f + k);
-    for (int a = 0; a < 2; ++a) accg[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ag[a], bg, accg[a], 0, 0, 0);
-    if constexpr (GLU) {
-      const bf16x8 bv = ld8(wv + k);
-      bf16x8 av[2];
-      for (int a = 0; a < 2; ++a) av[a] = ld8(xv + (long)rowA[a] * in_f + k);
-      for (int a = 0; a < 2; ++a) accv[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[a], bv, accv[a], 0, 0, 0);
+  // accumulators: [0] = the GEMM (gate GEMM for GLU), [1] = value GEMM (GLU only)
+  floatx16 acc[GLU ? 2 : 1][2][2];
+  static_for<0, (GLU ? 2 : 1)>([&](auto ss) {
+    static_for<0, 4>([&](auto tt) {
+      static_for<0, 16>([&](auto vv) { acc[decltype(ss)::value][decltype(tt)::value / 2][decltype(tt)::value % 2][decltype(vv)::value] = 0.f; });
+    });
+  });
+
+  auto compute = [&](int stage, auto set_) __attribute__((always_inline)) {
+    constexpr int set = decltype(set_)::value;
+    const uint16_t* sa = smem + stage * STAGE + (wr * 64 + i32) * kLdsRow + 8 * half;
+    const uint16_t* sb = smem + stage * STAGE + BM * kLdsRow + (wc * 64 + i32) * kLdsRow + 8 * half;
+    static_for<0, kBK / 16>([&](auto kk_) {
+      constexpr int kk = decltype(kk_)::value;
+      bf16x8 av[2], bv[2];
+      av[0] = ld8(sa + kk * 16);
+      av[1] = ld8(sa + 32 * kLdsRow + kk * 16);
+      bv[0] = ld8(sb + kk * 16);
+      bv[1] = ld8(sb + 32 * kLdsRow + kk * 16);
+      acc[set][0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[0], acc[set][0][0], 0, 0, 0);
+      acc[set][0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[1], acc[set][0][1], 0, 0, 0);
+      acc[set][1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[0], acc[set][1][0], 0, 0, 0);
+      acc[set][1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[1], acc[set][1][1], 0, 0, 0);
+    });
+  };
+
+  // NSTAGE == 2: double-buffered LDS, one barrier per chunk.  NSTAGE == 1: one LDS buffer and the next
+  // chunk parked in registers (two barriers per chunk, but half the LDS, so more workgroups per CU
+  // keep more loads in flight).
+  auto step = [&](int c, auto set_) __attribute__((always_inline)) {
+    if (c + 1 < nchunks) gload(c + 1);
+    compute(NSTAGE == 2 ? (c & 1) : 0, set_);
+    if constexpr (NSTAGE == 1) __syncthreads();
+    if (c + 1 < nchunks) sstore(NSTAGE == 2 ? ((c + 1) & 1) : 0);
+    __syncthreads();
+  };
+  gload(0);
+  sstore(0);
+  __syncthreads();
+  for (int c = 0; c < kchunks; ++c) step(c, ic<0>{});                 // first (or only) GEMM
+  if constexpr (GLU)
+    for (int c = kchunks; c < nchunks; ++c) step(c, ic<1>{});         // value GEMM
+
+  // ---- epilogue: tile -> LDS (fp32) -> coalesced rows, EP passes of BM / EP rows each ----
+  constexpr int OROW = BN + 4;                          // padded fp32 row
+  constexpr int EP = (WR == 4) ? 2 : 1;
+  constexpr int EROWS = BM / EP;
+  constexpr int TPR = BN / 4, RPI = 256 / TPR;          // each thread moves 4 consecutive columns
+  const int cq = (tid % TPR) * 4;
+  float4 bq = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (!GLU && bias) bq = *reinterpret_cast<const float4*>(bias + n0 + cq);
+  for (int ep = 0; ep < EP; ++ep) {
+    if (wr / (WR / EP) == ep) {
+      float* so = reinterpret_cast<float*>(smem) + ((wr % (WR / EP)) * 64 + 4 * half) * OROW + wc * 64 + i32;
+      static_for<0, 4>([&](auto tt) {
+        constexpr int t = decltype(tt)::value, a = t / 2, b = t % 2;
+        static_for<0, 16>([&](auto vv) {
+          constexpr int v = decltype(vv)::value;
+          float val = acc[0][a][b][v];
+          if constexpr (GLU) val = gelu_erf(val) * acc[GLU ? 1 : 0][a][b][v];
+          so[(32 * a + 8 * (v >> 2) + (v & 3)) * OROW + 32 * b] = val;
+        });
+      });
     }
-  }
-
-  const int col = n0 + i32;
-  const float bcol = (!GLU && bias) ? bias[col] : 0.f;
-  for (int a = 0; a < 2; ++a)
-    for (int v = 0; v < 16; ++v) {
-      const int r = m0 + 32 * a + 8 * (v >> 2) + 4 * half + (v & 3);
-      if (r >= M) continue;
-      float val;
-      if constexpr (GLU) {
-        val = gelu_erf(accg[a][v]) * accv[a][v];
-      } else {
-        val = accg[a][v] + bcol;
-        if (resid) val += bf16_to_f32(resid[(long)r * out_cols + col]);
+    __syncthreads();
+    const float* srow = reinterpret_cast<const float*>(smem) + cq;
+    for (int r = tid / TPR; r < EROWS; r += RPI) {
+      const int row = m0 + ep * EROWS + r;
+      if (row >= M) break;
+      float4 v4 = *reinterpret_cast<const float4*>(srow + r * OROW);
+      const long o = (long)row * out_cols + n0 + cq;
+      if constexpr (!GLU) {
+        v4.x += bq.x; v4.y += bq.y; v4.z += bq.z; v4.w += bq.w;
+        if (resid) {
+          const uint2 rr = *reinterpret_cast<const uint2*>(resid + o);
+          v4.x += __uint_as_float(rr.x << 16); v4.y += __uint_as_float(rr.x & 0xffff0000u);
+          v4.z += __uint_as_float(rr.y << 16); v4.w += __uint_as_float(rr.y & 0xffff0000u);
+        }
       }
-      if constexpr (sizeof(OUT) == 2) out[(long)r * out_cols + col] = f32_to_bf16(val);
-      else out[(long)r * out_cols + col] = val;
+      if constexpr (sizeof(OUT) == 2) {
+        uint2 pk;
+        pk.x = pack_bf16x2(v4.x, v4.y);
+        pk.y = pack_bf16x2(v4.z, v4.w);
+        *reinterpret_cast<uint2*>(out + o) = pk;
+      } else {
+        *reinterpret_cast<float4*>(out + o) = v4;
+      }
     }
+    if (ep + 1 < EP) __syncthreads();
+  }
+}
+
+template <int WR, int WC, bool GLU, typename OUT, int NSTAGE>
+static int launch_blockdiag(const void* x, const void* w, const float* bias, const void* resid, void* out, int M,
+                            int nb, int p, int q, int out_cols, hipStream_t stream) {
+  constexpr int BM = 64 * WR, BN = 64 * WC;
+  size_t lds = (size_t)NSTAGE * (BM + BN) * kLdsRow * sizeof(uint16_t);
+  const size_t epi = (size_t)(BM / (WR == 4 ? 2 : 1)) * (BN + 4) * sizeof(float);
+  if (epi > lds) lds = epi;
+  auto kern = blockdiag_kernel<WR, WC, GLU, OUT, NSTAGE>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(blockdiag): %s", hipGetErrorString(e));
+  }
+  dim3 grid(((M + BM - 1) / BM) * (out_cols / BN));
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, (const uint16_t*)x, (const uint16_t*)w, bias,
+                     (const uint16_t*)resid, (OUT*)out, M, nb, p, q);
+  return check_launch("blockdiag");
 }
 
 // LayerNorm over the last dimension of x (M, d) fp32, eps inside the square root.
-// Workgroup = 256 threads handles 64 rows: phase 1 one wave per row (16 rows per wave) writes the
-// row-major outputs and keeps mean / rstd in LDS; phase 2 re-reads the (cache-resident) rows with
-// lanes along the token axis and writes the channel-major copy with 256-byte stores.
-// d % 64 == 0, d <= 64 * kMaxPerLane.
-constexpr int kMaxPerLane = 32;
-__global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
-                                                        const float* __restrict__ beta, float eps,
-                                                        float* __restrict__ out_f32,       // (M, d) or null
-                                                        uint16_t* __restrict__ out_bf16,   // (M, d) or null
-                                                        float* __restrict__ out_t,         // (d, M) or null
-                                                        int M, int d) {
+// Workgroup = 16 waves handles 64 rows.  Phase 1: each wave normalises 4 rows at once (all loads in
+// flight together), writes the row-major outputs and leaves mean / rstd in LDS.  Phase 2 re-reads the
+// (cache-resident) rows with lanes along the token axis and writes the channel-major copy with
+// 256-byte stores.  PER = d / 64 values per lane.
+template <int PER>
+__global__ __launch_bounds__(1024) void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                         const float* __restrict__ beta, float eps,
+                                                         float* __restrict__ out_f32,       // (M, d) or null
+                                                         uint16_t* __restrict__ out_bf16,   // (M, d) or null
+                                                         float* __restrict__ out_t,         // (d, M) or null
+                                                         int M) {
+  constexpr int d = 64 * PER;
   __shared__ float s_mean[64], s_rstd[64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int m0 = blockIdx.x * 64;
-  const int per = d / 64;
-  for (int rr = 0; rr < 16; ++rr) {
-    const int rloc = wave * 16 + rr;
-    const int m = m0 + rloc;
-    if (m >= M) {
-      if (lane == 0) { s_mean[rloc] = 0.f; s_rstd[rloc] = 0.f; }
-      continue;
-    }
-    const float* xr = x + (long)m * d;
-    float v[kMaxPerLane];
-    float sum = 0.f;
-#pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i)
-      if (i < per) { v[i] = xr[lane + 64 * i]; sum += v[i]; }
-    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-    const float mean = sum / (float)d;
-    float sq = 0.f;
-#pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i)
-      if (i < per) { const float c = v[i] - mean; sq += c * c; }
-    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
-    const float rstd = rsqrtf(sq / (float)d + eps);
-    if (lane == 0) { s_mean[rloc] = mean; s_rstd[rloc] = rstd; }
-#pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i)
-      if (i < per) {
-        const int c = lane + 64 * i;
-        const float o = (v[i] - mean) * rstd * gamma[c] + beta[c];
-        if (out_f32) out_f32[(long)m * d + c] = o;
-        if (out_bf16) out_bf16[(long)m * d + c] = f32_to_bf16(o);
+  {
+    float v[4][PER];
+    float sum[4], sq[4];
+    static_for<0, 4>([&](auto rr_) {
+      constexpr int rr = decltype(rr_)::value;
+      int m = m0 + wave * 4 + rr;
+      m = m < M ? m : M - 1;
+      const float* xr = x + (long)m * d;
+      static_for<0, PER>([&](auto ii) { v[rr][decltype(ii)::value] = xr[lane + 64 * decltype(ii)::value]; });
+    });
+    float g[PER], bt[PER];
+    static_for<0, PER>([&](auto ii) {
+      g[decltype(ii)::value] = gamma[lane + 64 * decltype(ii)::value];
+      bt[decltype(ii)::value] = beta[lane + 64 * decltype(ii)::value];
+    });
+    static_for<0, 4>([&](auto rr_) {
+      constexpr int rr = decltype(rr_)::value;
+      float s = 0.f;
+      static_for<0, PER>([&](auto ii) { s += v[rr][decltype(ii)::value]; });
+      sum[rr] = s;
+    });
+    for (int o = 32; o > 0; o >>= 1)
+      static_for<0, 4>([&](auto rr_) { sum[decltype(rr_)::value] += __shfl_xor(sum[decltype(rr_)::value], o); });
+    static_for<0, 4>([&](auto rr_) {
+      constexpr int rr = decltype(rr_)::value;
+      sum[rr] *= (1.0f / (float)d);
+      float s = 0.f;
+      static_for<0, PER>([&](auto ii) {
+        const float c = v[rr][decltype(ii)::value] - sum[rr];
+        s += c * c;
+      });
+      sq[rr] = s;
+    });
+    for (int o = 32; o > 0; o >>= 1)
+      static_for<0, 4>([&](auto rr_) { sq[decltype(rr_)::value] += __shfl_xor(sq[decltype(rr_)::value], o); });
+    static_for<0, 4>([&](auto rr_) {
+      constexpr int rr = decltype(rr_)::value;
+      const int m = m0 + wave * 4 + rr;
+      const float mean = sum[rr];
+      const float rstd = rsqrtf(sq[rr] * (1.0f / (float)d) + eps);
+      if (lane == 0) { s_mean[wave * 4 + rr] = mean; s_rstd[wave * 4 + rr] = rstd; }
+      if (m < M) {
+        static_for<0, PER>([&](auto ii) {
+          constexpr int i = decltype(ii)::value;
+          const float o = (v[rr][i] - mean) * rstd * g[i] + bt[i];
+          if (out_f32) out_f32[(long)m * d + lane + 64 * i] = o;
+          if (out_bf16) out_bf16[(long)m * d + lane + 64 * i] = f32_to_bf16(o);
+        });
       }
+    });
   }
   if (!out_t) return;
   __syncthreads();
@@ -147,16 +313,16 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict_
   const bool ok = m < M;
   const float mean = s_mean[lane], rstd = s_rstd[lane];
   const float* xr = x + (long)(ok ? m : M - 1) * d;
-  for (int c0 = wave * 16; c0 < d; c0 += 64) {       // 16 channels per wave per step
-    float4 q[4];
-    for (int j = 0; j < 4; ++j) q[j] = *reinterpret_cast<const float4*>(xr + c0 + 4 * j);
-    const float vals[16] = {q[0].x, q[0].y, q[0].z, q[0].w, q[1].x, q[1].y, q[1].z, q[1].w,
-                            q[2].x, q[2].y, q[2].z, q[2].w, q[3].x, q[3].y, q[3].z, q[3].w};
-    if (ok)
-      for (int j = 0; j < 16; ++j) {
-        const int c = c0 + j;
-        out_t[(long)c * M + m] = (vals[j] - mean) * rstd * gamma[c] + beta[c];
-      }
+  for (int c0 = wave * 4; c0 < d; c0 += 64) {        // 4 channels per wave per step
+    const float4 q = *reinterpret_cast<const float4*>(xr + c0);
+    const float4 g4 = *reinterpret_cast<const float4*>(gamma + c0);
+    const float4 b4 = *reinterpret_cast<const float4*>(beta + c0);
+    if (ok) {
+      out_t[(long)(c0 + 0) * M + m] = (q.x - mean) * rstd * g4.x + b4.x;
+      out_t[(long)(c0 + 1) * M + m] = (q.y - mean) * rstd * g4.y + b4.y;
+      out_t[(long)(c0 + 2) * M + m] = (q.z - mean) * rstd * g4.z + b4.z;
+      out_t[(long)(c0 + 3) * M + m] = (q.w - mean) * rstd * g4.w + b4.w;
+    }
   }
 }
 
@@ -166,7 +332,7 @@ using namespace m2;
 
 static int check_blockdiag(const char* who, int M, int nb, int p, int q, bool glu) {
   if (M <= 0 || nb <= 0 || p <= 0 || q <= 0) return set_error(M2_ERR_ARG, "%s: sizes must be positive (M=%d nb=%d p=%d q=%d)", who, M, nb, p, q);
-  if (p % 16 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: in_features/nblocks=%d must be a multiple of 16", who, p);
+  if (p % 64 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: in_features/nblocks=%d must be a multiple of 64", who, p);
   if (q % 64 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: out_features/nblocks=%d must be a multiple of 64", who, q);
   if (glu && nb % 2 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: GLU pairing needs an even number of blocks, got %d", who, nb);
   return M2_OK;
@@ -181,10 +347,9 @@ extern "C" int m2_blockdiag_glu_fwd(const void* x, const void* w, void* out, int
   const int p = in_features / nblocks, q = 2 * intermediate / nblocks;
   int rc = check_blockdiag("m2_blockdiag_glu_fwd", M, nblocks, p, q, true);
   if (rc) return rc;
-  dim3 grid((M + 127) / 128, intermediate / 64);
-  hipLaunchKernelGGL((blockdiag_kernel<true, uint16_t>), grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x,
-                     (const uint16_t*)w, (const float*)nullptr, (const uint16_t*)nullptr, (uint16_t*)out, M, nblocks, p, q);
-  return check_launch("blockdiag_glu");
+  if (q % 128 == 0)
+    return launch_blockdiag<2, 2, true, uint16_t, 2>(x, w, nullptr, nullptr, out, M, nblocks, p, q, intermediate, (hipStream_t)stream);
+  return launch_blockdiag<4, 1, true, uint16_t, 2>(x, w, nullptr, nullptr, out, M, nblocks, p, q, intermediate, (hipStream_t)stream);
 }
 
 extern "C" int m2_blockdiag_linear_fwd(const void* x, const void* w, const float* bias, const void* residual,
@@ -199,23 +364,33 @@ extern "C" int m2_blockdiag_linear_fwd(const void* x, const void* w, const float
   const int p = in_features / nblocks, q = out_features / nblocks;
   int rc = check_blockdiag("m2_blockdiag_linear_fwd", M, nblocks, p, q, false);
   if (rc) return rc;
-  dim3 grid((M + 127) / 128, out_features / 64);
+  hipStream_t st = (hipStream_t)stream;
+  const bool wide = q % 128 == 0;
   if (out_dtype == M2_DTYPE_F32)
-    hipLaunchKernelGGL((blockdiag_kernel<false, float>), grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x,
-                       (const uint16_t*)w, bias, (const uint16_t*)residual, (float*)out, M, nblocks, p, q);
-  else
-    hipLaunchKernelGGL((blockdiag_kernel<false, uint16_t>), grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x,
-                       (const uint16_t*)w, bias, (const uint16_t*)residual, (uint16_t*)out, M, nblocks, p, q);
-  return check_launch("blockdiag_linear");
+    return wide ? launch_blockdiag<2, 2, false, float, 1>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st)
+                : launch_blockdiag<4, 1, false, float, 1>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st);
+  return wide ? launch_blockdiag<2, 2, false, uint16_t, 1>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st)
+              : launch_blockdiag<4, 1, false, uint16_t, 1>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st);
 }
 
 extern "C" int m2_layernorm_fwd(const float* x, const float* gamma, const float* beta, float eps, float* out_f32,
                                 void* out_bf16, float* out_channel_major, int M, int d, void* stream) {
   if (!x || !gamma || !beta) return set_error(M2_ERR_ARG, "m2_layernorm_fwd: null pointer");
-  if (M <= 0 || d <= 0 || d % 64 != 0 || d > 64 * kMaxPerLane)
-    return set_error(M2_ERR_UNSUPPORTED, "m2_layernorm_fwd: need M > 0 and d a multiple of 64 up to %d (M=%d d=%d)",
-                     64 * kMaxPerLane, M, d);
-  hipLaunchKernelGGL(layernorm_kernel, dim3((M + 63) / 64), dim3(256), 0, (hipStream_t)stream, x, gamma, beta, eps,
-                     out_f32, (uint16_t*)out_bf16, out_channel_major, M, d);
+  if (M <= 0 || d <= 0 || d % 64 != 0 || d > 2048)
+    return set_error(M2_ERR_UNSUPPORTED, "m2_layernorm_fwd: need M > 0 and d a multiple of 64 up to 2048 (M=%d d=%d)", M, d);
+  dim3 grid((M + 63) / 64);
+  hipStream_t st = (hipStream_t)stream;
+  uint16_t* o16 = (uint16_t*)out_bf16;
+  switch (d / 64) {
+#define LN_CASE(P)                                                                                                    \
+  case P:                                                                                                             \
+    hipLaunchKernelGGL(layernorm_kernel<P>, grid, dim3(1024), 0, st, x, gamma, beta, eps, out_f32, o16, out_channel_major, M); \
+    break;
+    LN_CASE(1) LN_CASE(2) LN_CASE(3) LN_CASE(4) LN_CASE(5) LN_CASE(6) LN_CASE(7) LN_CASE(8) LN_CASE(9) LN_CASE(10) LN_CASE(11)
+    LN_CASE(12) LN_CASE(13) LN_CASE(14) LN_CASE(15) LN_CASE(16) LN_CASE(17) LN_CASE(18) LN_CASE(19) LN_CASE(20) LN_CASE(21)
+    LN_CASE(22) LN_CASE(23) LN_CASE(24) LN_CASE(25) LN_CASE(26) LN_CASE(27) LN_CASE(28) LN_CASE(29) LN_CASE(30) LN_CASE(31)
+    LN_CASE(32)
+#undef LN_CASE
+  }
   return check_launch("layernorm");
 }

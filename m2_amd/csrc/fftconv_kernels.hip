@@ -311,7 +311,6 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
   const int tid = threadIdx.x;
   const int rloc = tid / T, t = tid % T;
   float2* row = lds + rloc * P::ROW_LDS;
-  const int nrows = d * B;
   const int n0 = 8 * t;
 
   cf wb1[16 / P::R1], wb2[16 / P::R2], wb3[16 / P::R3];
@@ -321,11 +320,16 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
   int g, g2;
   paired_groups<P>(t, g, g2);
 
-  for (int r0 = blockIdx.x * P::RPW; r0 < nrows; r0 += gridDim.x * P::RPW) {
-    const int r = r0 + rloc;
-    const bool valid = r < nrows;
-    const int rr = valid ? r : nrows - 1;
-    const int c = rr / B, b = rr % B;
+  // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each).  XCD e takes the channels
+  // c = e (mod 8) and runs the B rows of a channel on neighbouring workgroups at the same time, so a
+  // channel's spectrum is fetched into that L2 once and shared.  (d % 8 == 0 is checked by the host.)
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+  const int rows_per_xcd = (d >> 3) * B;
+  for (int j0 = slot * P::RPW; j0 < rows_per_xcd; j0 += slots * P::RPW) {
+    const int j = j0 + rloc;
+    const bool valid = j < rows_per_xcd;
+    const int jj = valid ? j : rows_per_xcd - 1;
+    const int c = (jj / B) * 8 + xcd, b = jj % B;
 
     // ---- prologue: 8 consecutive time steps per thread: short conv, gate, stage z = a + i u in LDS ----
     float gate[8];
@@ -544,11 +548,12 @@ static int launch_mixer_core(const void* xproj, const float* u, const float* sw,
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(mixer_core): %s", hipGetErrorString(e));
   }
-  const int nrows = d * B;
-  const int wgs_needed = (nrows + P::RPW - 1) / P::RPW;
+  const int rows_per_xcd = (d / 8) * B;
+  const int slots_needed = (rows_per_xcd + P::RPW - 1) / P::RPW;
   const int per_cu = (int)((160 * 1024) / lds_bytes) < 1 ? 1 : (int)((160 * 1024) / lds_bytes);
-  int grid = num_cus() * (per_cu > 8 ? 8 : per_cu);
-  if (grid > wgs_needed) grid = wgs_needed;
+  int slots = (num_cus() / 8) * (per_cu > 8 ? 8 : per_cu);          // workgroups per XCD
+  if (slots > slots_needed) slots = slots_needed;
+  const int grid = 8 * slots;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(P::WG), lds_bytes, stream, (const ACT*)xproj, u, sw, sb,
                      (const float4*)spec, (ACT*)y, B, d);
   return check_launch("mixer_core");
@@ -612,7 +617,7 @@ extern "C" int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, co
 extern "C" int m2_mixer_core_fwd(const void* xproj, const float* u, const float* short_w, const float* short_b,
                                  const float* spec, void* y, int B, int L, int d, int act_dtype, void* stream) {
   if (!xproj || !short_w || !short_b || !spec || !y) return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: null pointer");
-  if (B <= 0 || d <= 0) return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: bad sizes B=%d d=%d", B, d);
+  if (B <= 0 || d <= 0 || d % 8 != 0) return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: need B > 0 and d a positive multiple of 8 (B=%d d=%d)", B, d);
   if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
     return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
   if (!m2_fftconv_supported_seqlen(L))
@@ -634,7 +639,7 @@ extern "C" int m2_mixer_core_fwd(const void* xproj, const float* u, const float*
 extern "C" int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, int L, int d, int act_dtype,
                               void* stream) {
   if (!x || !spec || !y) return set_error(M2_ERR_ARG, "m2_fftconv_fwd: null pointer");
-  if (B <= 0 || d <= 0) return set_error(M2_ERR_ARG, "m2_fftconv_fwd: bad sizes B=%d d=%d", B, d);
+  if (B <= 0 || d <= 0 || d % 8 != 0) return set_error(M2_ERR_ARG, "m2_fftconv_fwd: need B > 0 and d a positive multiple of 8 (B=%d d=%d)", B, d);
   if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
     return set_error(M2_ERR_ARG, "m2_fftconv_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
   if (!m2_fftconv_supported_seqlen(L))

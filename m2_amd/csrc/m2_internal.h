@@ -28,4 +28,16 @@ __host__ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
   return v.f;
 }
 
+// two floats -> packed bf16 pair (lo in bits 0..15), round to nearest even; one v_cvt_pk_bf16_f32 on the device
+__host__ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+#else
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+#endif
+}
+
 }  // namespace m2
