@@ -97,12 +97,15 @@ int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, const float* 
  *            a = sc(v) * sc(x1),  sc = depthwise 3-tap causal conv + bias (cross-correlation,
  *            out[t] = bias + w0 in[t-2] + w1 in[t-1] + w2 in[t]);  D1, D2 are already inside spec.
  * xproj  (3d, B, L)  in_linear output, CHANNEL-MAJOR, channels [0,d)=x1, [d,2d)=x2, [2d,3d)=v; act_dtype
+ * proj_bias (3d)     fp32, added to xproj as it is read (the in_linear bias, so the projection GEMM can
+ *                    run without a bias pass); NULL when xproj already contains it
  * u      (d, B, L)   fp32 layer input, channel-major; NULL when there is no residual long conv
  * short_w (3d, 3), short_b (3d)  fp32
  * spec   from m2_filter_spectrum_fwd with the same d and L
  * y      (d, B, L)   act_dtype (M2_DTYPE_F32 or M2_DTYPE_BF16); FFT arithmetic is fp32 either way */
-int m2_mixer_core_fwd(const void* xproj, const float* u, const float* short_w, const float* short_b,
-                      const float* spec, void* y, int B, int L, int d, int act_dtype, void* stream);
+int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, const float* u, const float* short_w,
+                      const float* short_b, const float* spec, void* y, int B, int L, int d, int act_dtype,
+                      void* stream);
 
 /* Plain long convolution y[c,b,:] = fftconv(x[c,b,:]; k1)[:L] + D1[c] x[c,b,:] with the first filter
  * of `spec` (HyenaFilter.forward on its own, bert/src/mm/hyena_utils.py:219-248).

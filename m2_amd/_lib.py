@@ -44,8 +44,8 @@ def _load() -> ctypes.CDLL:
     lib.m2_filter_spectrum_fwd.restype = c_int
     lib.m2_filter_spectrum_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]
     lib.m2_mixer_core_fwd.restype = c_int
-    lib.m2_mixer_core_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                      c_int, c_void_p]
+    lib.m2_mixer_core_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                      c_int, c_int, c_void_p]
     lib.m2_fftconv_fwd.restype = c_int
     lib.m2_fftconv_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
     lib.m2_blockdiag_glu_fwd.restype = c_int

@@ -256,30 +256,31 @@ __global__ __launch_bounds__(1024) void layernorm_kernel(const float* __restrict
   __shared__ float s_mean[64], s_rstd[64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int m0 = blockIdx.x * 64;
-  {
-    float v[4][PER];
-    float sum[4], sq[4];
-    static_for<0, 4>([&](auto rr_) {
+  constexpr int RW = PER <= 16 ? 4 : 2;                 // rows in flight per wave (register budget of 128)
+  float g[PER], bt[PER];
+  static_for<0, PER>([&](auto ii) {
+    g[decltype(ii)::value] = gamma[lane + 64 * decltype(ii)::value];
+    bt[decltype(ii)::value] = beta[lane + 64 * decltype(ii)::value];
+  });
+  for (int rb = 0; rb < 4; rb += RW) {
+    float v[RW][PER];
+    float sum[RW], sq[RW];
+    static_for<0, RW>([&](auto rr_) {
       constexpr int rr = decltype(rr_)::value;
-      int m = m0 + wave * 4 + rr;
+      int m = m0 + wave * 4 + rb + rr;
       m = m < M ? m : M - 1;
       const float* xr = x + (long)m * d;
       static_for<0, PER>([&](auto ii) { v[rr][decltype(ii)::value] = xr[lane + 64 * decltype(ii)::value]; });
     });
-    float g[PER], bt[PER];
-    static_for<0, PER>([&](auto ii) {
-      g[decltype(ii)::value] = gamma[lane + 64 * decltype(ii)::value];
-      bt[decltype(ii)::value] = beta[lane + 64 * decltype(ii)::value];
-    });
-    static_for<0, 4>([&](auto rr_) {
+    static_for<0, RW>([&](auto rr_) {
       constexpr int rr = decltype(rr_)::value;
       float s = 0.f;
       static_for<0, PER>([&](auto ii) { s += v[rr][decltype(ii)::value]; });
       sum[rr] = s;
     });
     for (int o = 32; o > 0; o >>= 1)
-      static_for<0, 4>([&](auto rr_) { sum[decltype(rr_)::value] += __shfl_xor(sum[decltype(rr_)::value], o); });
-    static_for<0, 4>([&](auto rr_) {
+      static_for<0, RW>([&](auto rr_) { sum[decltype(rr_)::value] += __shfl_xor(sum[decltype(rr_)::value], o); });
+    static_for<0, RW>([&](auto rr_) {
       constexpr int rr = decltype(rr_)::value;
       sum[rr] *= (1.0f / (float)d);
       float s = 0.f;
@@ -290,13 +291,13 @@ __global__ __launch_bounds__(1024) void layernorm_kernel(const float* __restrict
       sq[rr] = s;
     });
     for (int o = 32; o > 0; o >>= 1)
-      static_for<0, 4>([&](auto rr_) { sq[decltype(rr_)::value] += __shfl_xor(sq[decltype(rr_)::value], o); });
-    static_for<0, 4>([&](auto rr_) {
+      static_for<0, RW>([&](auto rr_) { sq[decltype(rr_)::value] += __shfl_xor(sq[decltype(rr_)::value], o); });
+    static_for<0, RW>([&](auto rr_) {
       constexpr int rr = decltype(rr_)::value;
-      const int m = m0 + wave * 4 + rr;
+      const int m = m0 + wave * 4 + rb + rr;
       const float mean = sum[rr];
       const float rstd = rsqrtf(sq[rr] * (1.0f / (float)d) + eps);
-      if (lane == 0) { s_mean[wave * 4 + rr] = mean; s_rstd[wave * 4 + rr] = rstd; }
+      if (lane == 0) { s_mean[wave * 4 + rb + rr] = mean; s_rstd[wave * 4 + rb + rr] = rstd; }
       if (m < M) {
         static_for<0, PER>([&](auto ii) {
           constexpr int i = decltype(ii)::value;

@@ -239,24 +239,30 @@ __device__ __forceinline__ void pair_multiply(cf& za, cf& zb, float4 K) {
 // ------------------------------------------------------------------------------------------
 // 8 consecutive activations starting at element n0 (n0 % 8 == 0) plus the two before them, as fp32:
 // out[0], out[1] = in[n0-2], in[n0-1] (zero when n0 == 0), out[2..10) = in[n0 .. n0+8).
-__device__ __forceinline__ void load10(const float* p, int n0, float (&o)[10]) {
+// `add` is added to every element that exists (the two before n0 == 0 stay zero: that is the
+// convolution's zero padding, which sits outside the biased signal).
+__device__ __forceinline__ void load10(const float* p, int n0, float add, float (&o)[10]) {
   const float4 a = *reinterpret_cast<const float4*>(p + n0);
   const float4 b = *reinterpret_cast<const float4*>(p + n0 + 4);
-  float2 h = make_float2(0.f, 0.f);
-  if (n0 > 0) h = *reinterpret_cast<const float2*>(p + n0 - 2);
-  o[0] = h.x; o[1] = h.y;
-  o[2] = a.x; o[3] = a.y; o[4] = a.z; o[5] = a.w;
-  o[6] = b.x; o[7] = b.y; o[8] = b.z; o[9] = b.w;
+  o[0] = 0.f; o[1] = 0.f;
+  if (n0 > 0) {
+    const float2 h = *reinterpret_cast<const float2*>(p + n0 - 2);
+    o[0] = h.x + add; o[1] = h.y + add;
+  }
+  o[2] = a.x + add; o[3] = a.y + add; o[4] = a.z + add; o[5] = a.w + add;
+  o[6] = b.x + add; o[7] = b.y + add; o[8] = b.z + add; o[9] = b.w + add;
 }
-__device__ __forceinline__ void load10(const uint16_t* p, int n0, float (&o)[10]) {
+__device__ __forceinline__ void load10(const uint16_t* p, int n0, float add, float (&o)[10]) {
   const uint4 a = *reinterpret_cast<const uint4*>(p + n0);
-  uint32_t h = 0;
-  if (n0 > 0) h = *reinterpret_cast<const uint32_t*>(p + n0 - 2);
-  o[0] = __uint_as_float(h << 16); o[1] = __uint_as_float(h & 0xffff0000u);
-  o[2] = __uint_as_float(a.x << 16); o[3] = __uint_as_float(a.x & 0xffff0000u);
-  o[4] = __uint_as_float(a.y << 16); o[5] = __uint_as_float(a.y & 0xffff0000u);
-  o[6] = __uint_as_float(a.z << 16); o[7] = __uint_as_float(a.z & 0xffff0000u);
-  o[8] = __uint_as_float(a.w << 16); o[9] = __uint_as_float(a.w & 0xffff0000u);
+  o[0] = 0.f; o[1] = 0.f;
+  if (n0 > 0) {
+    const uint32_t h = *reinterpret_cast<const uint32_t*>(p + n0 - 2);
+    o[0] = __uint_as_float(h << 16) + add; o[1] = __uint_as_float(h & 0xffff0000u) + add;
+  }
+  o[2] = __uint_as_float(a.x << 16) + add; o[3] = __uint_as_float(a.x & 0xffff0000u) + add;
+  o[4] = __uint_as_float(a.y << 16) + add; o[5] = __uint_as_float(a.y & 0xffff0000u) + add;
+  o[6] = __uint_as_float(a.z << 16) + add; o[7] = __uint_as_float(a.z & 0xffff0000u) + add;
+  o[8] = __uint_as_float(a.w << 16) + add; o[9] = __uint_as_float(a.w & 0xffff0000u) + add;
 }
 __device__ __forceinline__ void store8(float* p, int n0, const float (&v)[8]) {
   *reinterpret_cast<float4*>(p + n0) = make_float4(v[0], v[1], v[2], v[3]);
@@ -303,6 +309,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
     const float* __restrict__ uin,      // (d, B, L)   layer input, channel-major (may be null)
     const float* __restrict__ sw,       // (3d, 3)     short-conv taps; null = plain convolution of a (d, B, L) input
     const float* __restrict__ sb,       // (3d)        short-conv bias
+    const float* __restrict__ pbias,    // (3d)        bias of the in-projection, added to xproj on load (may be null)
     const float4* __restrict__ spec,    // (d, 8, T)   native-order spectra
     ACT* __restrict__ y,                // (d, B, L)
     int B, int d) {
@@ -337,7 +344,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
       float in[10], a[8];
       if (sw) {
         const float* w = sw + (long)c * 3;
-        load10(xproj + ((long)(0 * d + c) * B + b) * L, n0, in);
+        load10(xproj + ((long)(0 * d + c) * B + b) * L, n0, pbias ? pbias[c] : 0.f, in);
         {
           const float w0 = w[0], w1 = w[1], w2 = w[2], bb = sb[c];
           static_for<0, 8>([&](auto jj) {
@@ -345,7 +352,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
             a[j] = bb + w0 * in[j] + w1 * in[j + 1] + w2 * in[j + 2];
           });
         }
-        load10(xproj + ((long)(2 * d + c) * B + b) * L, n0, in);
+        load10(xproj + ((long)(2 * d + c) * B + b) * L, n0, pbias ? pbias[2 * d + c] : 0.f, in);
         {
           const float w0 = w[6 * (long)d + 0], w1 = w[6 * (long)d + 1], w2 = w[6 * (long)d + 2], bb = sb[2 * d + c];
           static_for<0, 8>([&](auto jj) {
@@ -353,7 +360,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
             a[j] *= bb + w0 * in[j] + w1 * in[j + 1] + w2 * in[j + 2];
           });
         }
-        load10(xproj + ((long)(1 * d + c) * B + b) * L, n0, in);
+        load10(xproj + ((long)(1 * d + c) * B + b) * L, n0, pbias ? pbias[d + c] : 0.f, in);
         {
           const float w0 = w[3 * (long)d + 0], w1 = w[3 * (long)d + 1], w2 = w[3 * (long)d + 2], bb = sb[d + c];
           static_for<0, 8>([&](auto jj) {
@@ -363,7 +370,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
         }
       } else {
         // plain long convolution: xproj is a single (d, B, L) signal, no short conv, no gates
-        load10(xproj + ((long)c * B + b) * L, n0, in);
+        load10(xproj + ((long)c * B + b) * L, n0, 0.f, in);
         static_for<0, 8>([&](auto jj) {
           constexpr int j = decltype(jj)::value;
           a[j] = in[j + 2];
@@ -540,8 +547,8 @@ __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
 // host-side dispatch
 // ------------------------------------------------------------------------------------------
 template <class P, typename ACT>
-static int launch_mixer_core(const void* xproj, const float* u, const float* sw, const float* sb, const float* spec,
-                             void* y, int B, int d, hipStream_t stream) {
+static int launch_mixer_core(const void* xproj, const float* u, const float* sw, const float* sb, const float* pbias,
+                             const float* spec, void* y, int B, int d, hipStream_t stream) {
   const size_t lds_bytes = (size_t)P::RPW * P::ROW_LDS * sizeof(float2);
   auto kern = mixer_core_kernel<P, ACT>;
   if (lds_bytes > 64 * 1024) {
@@ -554,7 +561,7 @@ static int launch_mixer_core(const void* xproj, const float* u, const float* sw,
   int slots = (num_cus() / 8) * (per_cu > 8 ? 8 : per_cu);          // workgroups per XCD
   if (slots > slots_needed) slots = slots_needed;
   const int grid = 8 * slots;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(P::WG), lds_bytes, stream, (const ACT*)xproj, u, sw, sb,
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(P::WG), lds_bytes, stream, (const ACT*)xproj, u, sw, sb, pbias,
                      (const float4*)spec, (ACT*)y, B, d);
   return check_launch("mixer_core");
 }
@@ -614,8 +621,9 @@ extern "C" int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, co
   return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: no plan for L=%d", L);
 }
 
-extern "C" int m2_mixer_core_fwd(const void* xproj, const float* u, const float* short_w, const float* short_b,
-                                 const float* spec, void* y, int B, int L, int d, int act_dtype, void* stream) {
+extern "C" int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, const float* u, const float* short_w,
+                                 const float* short_b, const float* spec, void* y, int B, int L, int d, int act_dtype,
+                                 void* stream) {
   if (!xproj || !short_w || !short_b || !spec || !y) return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: null pointer");
   if (B <= 0 || d <= 0 || d % 8 != 0) return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: need B > 0 and d a positive multiple of 8 (B=%d d=%d)", B, d);
   if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
@@ -628,8 +636,8 @@ extern "C" int m2_mixer_core_fwd(const void* xproj, const float* u, const float*
 #define X(LOGN, R1, R2, R3)                                                                                       \
   case LOGN:                                                                                                      \
     return act_dtype == M2_DTYPE_F32                                                                              \
-               ? launch_mixer_core<Plan<LOGN, R1, R2, R3>, float>(xproj, u, short_w, short_b, spec, y, B, d, s) \
-               : launch_mixer_core<Plan<LOGN, R1, R2, R3>, uint16_t>(xproj, u, short_w, short_b, spec, y, B, d, s);
+               ? launch_mixer_core<Plan<LOGN, R1, R2, R3>, float>(xproj, u, short_w, short_b, proj_bias, spec, y, B, d, s) \
+               : launch_mixer_core<Plan<LOGN, R1, R2, R3>, uint16_t>(xproj, u, short_w, short_b, proj_bias, spec, y, B, d, s);
     M2_FOR_EACH_PLAN(X)
 #undef X
   }
@@ -650,8 +658,8 @@ extern "C" int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, 
 #define X(LOGN, R1, R2, R3)                                                                                  \
   case LOGN:                                                                                                 \
     return act_dtype == M2_DTYPE_F32                                                                         \
-               ? launch_mixer_core<Plan<LOGN, R1, R2, R3>, float>(x, nullptr, nullptr, nullptr, spec, y, B, d, s) \
-               : launch_mixer_core<Plan<LOGN, R1, R2, R3>, uint16_t>(x, nullptr, nullptr, nullptr, spec, y, B, d, s);
+               ? launch_mixer_core<Plan<LOGN, R1, R2, R3>, float>(x, nullptr, nullptr, nullptr, nullptr, spec, y, B, d, s) \
+               : launch_mixer_core<Plan<LOGN, R1, R2, R3>, uint16_t>(x, nullptr, nullptr, nullptr, nullptr, spec, y, B, d, s);
     M2_FOR_EACH_PLAN(X)
 #undef X
   }

@@ -6,7 +6,7 @@ in the reference (bert/src/bert_layers.py:131-252 BertEmbeddings, :457-508 BertG
 layer so that no activation is transposed or re-read in between:
 
     h32 (M,d) f32, h16 (M,d) bf16, hT (d,M) f32   <- LayerNorm of the previous layer (three forms, one kernel)
-    xproj (3d,M) bf16 = W_in h16^T + b            library GEMM, channel-major output
+    xproj (3d,M) bf16 = W_in h16^T                library GEMM, channel-major output (bias added by K2)
     spec              = filter spectra            K1 (hidden MLP, projection+decay) + spectrum FFT
     y (d,M) bf16      = mixer core(xproj, hT)     K2
     a (M,d) bf16      = y^T W_out^T + b           library GEMM
@@ -136,10 +136,9 @@ class BertLayer(nn.Module):
         at = self.attention
         d = at.d_model
         w_in = at._cast("in_w", at.in_linear.weight, torch.bfloat16)
-        b_in = at._cast("in_b", at.in_linear.bias, torch.bfloat16)
         w_out = at._cast("out_w", at.out_linear.weight, torch.bfloat16)
         b_out = at._cast("out_b", at.out_linear.bias, torch.bfloat16)
-        xproj = torch.addmm(b_in.unsqueeze(1), w_in, h16.t())                        # (3d, M)
+        xproj = torch.mm(w_in, h16.t())                                              # (3d, M); bias added in the core
         y = at.core(xproj.view(3 * d, B, L), hT.view(d, B, L) if at.residual_long_conv else None, B, L)
         a16 = torch.addmm(b_out, y.view(d, B * L).t(), w_out.t())                    # (M, d)
         s = self.mlp.presum(a16)

@@ -78,12 +78,14 @@ class MonarchMixerSequenceMixing(nn.Module):
 
     def core(self, xproj: torch.Tensor, u_cm: Optional[torch.Tensor], B: int, L: int,
              spec: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Channel-major core: xproj (3d, B, L), u_cm (d, B, L) fp32 -> y (d, B, L)."""
+        """Channel-major core: xproj (3d, B, L) = in_linear.weight @ u^T WITHOUT the bias (the kernel adds
+        in_linear.bias as it loads), u_cm (d, B, L) fp32 -> y (d, B, L)."""
         if spec is None:
             spec = self.filter_spectrum(L)
         sw = self._cast("short_w", self.short_filter.weight, torch.float32).view(3 * self.d_model, 3)
         sb = self._cast("short_b", self.short_filter.bias, torch.float32)
-        return ops.mixer_core(xproj, u_cm, sw, sb, spec, B, L, self.d_model)
+        pb = self._cast("in_b32", self.in_linear.bias, torch.float32)
+        return ops.mixer_core(xproj, u_cm, sw, sb, spec, B, L, self.d_model, proj_bias=pb)
 
     # -- reference API -----------------------------------------------------------------------
     def forward(self, u, **kwargs):
@@ -96,11 +98,10 @@ class MonarchMixerSequenceMixing(nn.Module):
         act = torch.bfloat16 if low else torch.float32
         u2 = u.reshape(B * L, d)
         w_in = self._cast("in_w", self.in_linear.weight, act)
-        b_in = self._cast("in_b", self.in_linear.bias, act)
         w_out = self._cast("out_w", self.out_linear.weight, act)
         b_out = self._cast("out_b", self.out_linear.bias, act)
         with torch.autocast("cuda", enabled=False):
-            xproj = torch.addmm(b_in.unsqueeze(1), w_in, u2.to(act).t())              # (3d, B*L)
+            xproj = torch.mm(w_in, u2.to(act).t())                                      # (3d, B*L), bias added in the core
             u_cm = u2.float().t().contiguous() if self.residual_long_conv else None      # (d, B*L)
             y = self.core(xproj.view(3 * d, B, L), None if u_cm is None else u_cm.view(d, B, L), B, L)
             out = torch.addmm(b_out, y.view(d, B * L).t(), w_out.t())                   # (B*L, d)

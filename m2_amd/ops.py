@@ -111,10 +111,13 @@ def filter_spectrum(taps1: Tensor, taps2: Optional[Tensor], D1: Optional[Tensor]
 
 
 def mixer_core(xproj: Tensor, u: Optional[Tensor], short_w: Tensor, short_b: Tensor, spec: Tensor, B: int, L: int,
-               d: int, out: Optional[Tensor] = None) -> Tensor:
-    """y (d, B, L) from the channel-major in-projection (3d, B, L) and layer input (d, B, L)."""
+               d: int, out: Optional[Tensor] = None, proj_bias: Optional[Tensor] = None) -> Tensor:
+    """y (d, B, L) from the channel-major in-projection (3d, B, L) and layer input (d, B, L).
+    `proj_bias` (3d) fp32 is added to xproj on load (pass the in_linear bias when the GEMM ran without it)."""
     _require(xproj, "xproj", None, (3 * d, B, L))
     code = _act_code(xproj.dtype)
+    if proj_bias is not None:
+        _require(proj_bias, "proj_bias", torch.float32, (3 * d,))
     if u is not None:
         _require(u, "u", torch.float32, (d, B, L))
     _require(short_w, "short_w", torch.float32, (3 * d, 3))
@@ -124,8 +127,8 @@ def mixer_core(xproj: Tensor, u: Optional[Tensor], short_w: Tensor, short_b: Ten
         out = torch.empty(d, B, L, dtype=xproj.dtype, device=xproj.device)
     else:
         _require(out, "out", xproj.dtype, (d, B, L))
-    check(lib.m2_mixer_core_fwd(_ptr(xproj), _ptr(u), _ptr(short_w), _ptr(short_b), _ptr(spec), _ptr(out), B, L, d,
-                                code, _stream()))
+    check(lib.m2_mixer_core_fwd(_ptr(xproj), _ptr(proj_bias), _ptr(u), _ptr(short_w), _ptr(short_b), _ptr(spec),
+                                _ptr(out), B, L, d, code, _stream()))
     return out
 
 

@@ -40,12 +40,12 @@ def test_size_queries_and_argument_checks_without_gpu():
     assert lib.m2_filter_spectrum_bytes(768, 8192) == 768 * 8192 * 16
     assert lib.m2_hyena_filter_workspace_bytes(2, 8192, 128) == 2 * 2 * 8192 * 128 * 4
     # null pointers and unsupported sizes are refused before anything is launched
-    assert lib.m2_mixer_core_fwd(None, None, None, None, None, None, 1, 128, 64, 0, None) == -1
+    assert lib.m2_mixer_core_fwd(None, None, None, None, None, None, None, 1, 128, 64, 0, None) == -1
     assert b"null" in lib.m2_last_error()
     one = ctypes.c_void_p(16)
-    assert lib.m2_mixer_core_fwd(one, None, one, one, one, one, 1, 100, 64, 0, None) == -2
+    assert lib.m2_mixer_core_fwd(one, None, None, one, one, one, one, 1, 100, 64, 0, None) == -2
     assert b"L=100" in lib.m2_last_error()
-    assert lib.m2_mixer_core_fwd(one, None, one, one, one, one, 1, 128, 64, 7, None) == -1
+    assert lib.m2_mixer_core_fwd(one, None, None, one, one, one, one, 1, 128, 64, 7, None) == -1
     assert lib.m2_blockdiag_glu_fwd(one, one, one, 8, 768, 3072, 3, None) == -2
     assert lib.m2_blockdiag_linear_fwd(one, one, None, None, one, 8, 100, 64, 4, 1, None) == -2
     assert lib.m2_layernorm_fwd(one, one, one, 1e-12, None, None, None, 4, 100, None) == -2

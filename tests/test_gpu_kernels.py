@@ -72,9 +72,10 @@ def test_mixer_core(gpu, L, act):
     taps = [torch.randn(d, 2 * L, generator=g) * torch.exp(-4 * torch.minimum(t, 1 - t)) for _ in range(2)]
     D = [torch.randn(d, generator=g) for _ in range(2)]
     spec = ops.filter_spectrum(taps[0].to(gpu), taps[1].to(gpu), D[0].to(gpu), D[1].to(gpu))
-    y = ops.mixer_core(xproj.to(gpu), u.to(gpu), sw.to(gpu), sb.to(gpu), spec, B, L, d)
+    pb = torch.randn(3 * d, generator=g) * 0.3
+    y = ops.mixer_core(xproj.to(gpu), u.to(gpu), sw.to(gpu), sb.to(gpu), spec, B, L, d, proj_bias=pb.to(gpu))
     # oracle in float64 on the same (possibly bf16-rounded) inputs
-    x64 = xproj.double().permute(1, 0, 2)                      # (B, 3d, L)
+    x64 = (xproj.double() + pb.double()[:, None, None]).permute(1, 0, 2)      # (B, 3d, L)
     uc = O.short_conv(x64, sw.double().view(3 * d, 1, 3), sb.double())
     x1, x2, v = uc.split(d, dim=1)
     y1 = O.fftconv(v * x1, taps[0].double(), D[0].double()[None, :, None])
