@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Throughput of the M2-BERT-80M encoder forward on one MI355X, sequences per second.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c2|c5|c1] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c2|c4|c5] [--no-cpu-baseline]
 
 A step is one forward of embeddings + 12 Monarch-Mixer layers over one synthetic batch that is
 already resident in HBM (token ids on the GPU; filters are regenerated from the weights in every
@@ -39,6 +39,10 @@ def workload(name: str):
         cfg, B, pad = m2_amd.m2_bert_80m(128), 32, False
         label = "M2-BERT-80M encoder fwd, L=128, B=32 (config 1)"
         idx = 1
+    elif name == "c4":
+        cfg, B, pad = m2_amd.m2_bert_80m(32768), 1, False
+        label = "M2-BERT-80M encoder fwd, L=32768, B=1 (config 3)"
+        idx = 3
     elif name == "c5":
         cfg, B, pad = m2_amd.m2_bert_large(128, 24), 64, False
         label = "M2-BERT large 24x1536 encoder fwd, L=128, B=64 (config 4)"

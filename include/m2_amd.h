@@ -79,7 +79,8 @@ int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int 
  * native counterpart in the reference: flashmm.mm_block_fwd (csrc/flashmm/flash_mm.cpp:70-226).
  * ------------------------------------------------------------------------------------------- */
 
-/* 1 if sequence length L is supported by the LDS-resident FFT (2L a power of two in [256, 16384]). */
+/* 1 if sequence length L is supported: 2L a power of two in [256, 16384] (one LDS-resident FFT per
+ * row) or 2L = 65536 (four LDS-resident sub-transforms per row). */
 int m2_fftconv_supported_seqlen(int L);
 
 /* Bytes of the opaque spectrum buffer for d channels and sequence length L (both filters). */

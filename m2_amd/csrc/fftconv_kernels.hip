@@ -33,206 +33,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "fft_regs.h"
-#include "m2_internal.h"
+#include "fft_engine.h"
 
 namespace m2 {
-
-// ------------------------------------------------------------------------------------------
-// plan
-// ------------------------------------------------------------------------------------------
-template <int LOGN_, int R1_, int R2_, int R3_>
-struct Plan {
-  static constexpr int LOGN = LOGN_, N = 1 << LOGN_, L = N / 2;
-  static constexpr int E = 16, RP = 8;
-  static constexpr int R1 = R1_, R2 = R2_, R3 = R3_;
-  static constexpr int T = N / E;            // threads per row
-  static constexpr int M = N / RP;           // groups of 8 in the last pass
-  static constexpr int S1 = N / R1, S2 = S1 / R2, S3 = S2 / R3;
-  static constexpr int RL = (R3 > 1) ? R3 : R2;   // radix of the least significant digit of a group index
-  static constexpr int WG = T < 256 ? 256 : T;    // threads per workgroup
-  static constexpr int RPW = WG / T;              // rows per workgroup
-  static constexpr int ROW_LDS = N + (N >> 4);    // padded complex slots per row
-  static_assert(R1 * R2 * R3 * RP == N, "radices must multiply to N");
-  static_assert(S3 == RP, "last stride");
-  static_assert(R1 * R2 >= E, "passes after the first must share twiddles inside a thread");
-};
-
-__device__ __forceinline__ int phys(int pos) { return pos + (pos >> 4); }
-
-// Padded offset of logical offset `o` relative to a base position whose low four bits, added to
-// (o mod 16), stay below 16.  True for every access below: strides are multiples of 16, or 8 with a
-// base offset below 8, or consecutive runs of 8 that start at a multiple of 8.
-constexpr int poff(int o) { return o + (o >> 4); }
-
-__device__ __forceinline__ cf lds_get(const float2* p, int off) {
-  float2 v = p[off];
-  return {v.x, v.y};
-}
-__device__ __forceinline__ void lds_put(float2* p, int off, cf v) { p[off] = make_float2(v.re, v.im); }
-
-// exp(-2*pi*i*m/n), n a power of two
-__device__ __forceinline__ cf unit_root(int m, int n) {
-  float s, c;
-  sincospif(2.0f * (float)m / (float)n, &s, &c);
-  return {c, -s};
-}
-
-// ------------------------------------------------------------------------------------------
-// generic passes on the row held in LDS
-// ------------------------------------------------------------------------------------------
-// forward: registers hold natural-order inputs of E/R butterflies; butterfly, twiddle, store.
-template <class P, int R, int S, bool ZERO_UPPER>
-__device__ __forceinline__ void fwd_compute_store(cf (&x)[16], int t, float2* row, const cf (&wbase)[16 / R]) {
-  constexpr int NB = 16 / R;
-  static_for<0, NB>([&](auto ii) {
-    constexpr int i = decltype(ii)::value;
-    const int q = t + P::T * i;
-    const int b = q / S, m = q % S;
-    if constexpr (ZERO_UPPER) dif_zero_upper<R, i * R, 16>(x);
-    else dif<R, i * R, 16>(x);
-    cf p[R];
-    powers<R>(wbase[(S > P::T) ? i : 0], p);
-    float2* pb = row + phys(b * (S * R) + m);
-    constexpr int bits = ilog2(R);
-    static_for<0, R>([&](auto kk) {
-      constexpr int k = decltype(kk)::value;
-      cf v = x[i * R + bitrev(k, bits)];
-      if constexpr (k > 0) v = cmul(v, p[k]);
-      lds_put(pb, poff(k * S), v);
-    });
-  });
-}
-
-template <class P, int R, int S>
-__device__ __forceinline__ void fwd_load(cf (&x)[16], int t, const float2* row) {
-  constexpr int NB = 16 / R;
-  static_for<0, NB>([&](auto ii) {
-    constexpr int i = decltype(ii)::value;
-    const int q = t + P::T * i;
-    const int b = q / S, m = q % S;
-    const float2* pb = row + phys(b * (S * R) + m);
-    static_for<0, R>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      x[i * R + j] = lds_get(pb, poff(j * S));
-    });
-  });
-}
-
-// inverse: load digit k into bit-reversed register, conj twiddle, inverse butterfly (natural out)
-template <class P, int R, int S, bool LOWER_ONLY>
-__device__ __forceinline__ void inv_load_compute(cf (&x)[16], int t, const float2* row, const cf (&wbase)[16 / R]) {
-  constexpr int NB = 16 / R;
-  static_for<0, NB>([&](auto ii) {
-    constexpr int i = decltype(ii)::value;
-    const int q = t + P::T * i;
-    const int b = q / S, m = q % S;
-    cf p[R];
-    powers<R>(wbase[(S > P::T) ? i : 0], p);
-    const float2* pb = row + phys(b * (S * R) + m);
-    constexpr int bits = ilog2(R);
-    static_for<0, R>([&](auto kk) {
-      constexpr int k = decltype(kk)::value;
-      cf v = lds_get(pb, poff(k * S));
-      if constexpr (k > 0) v = cmulc(v, p[k]);
-      x[i * R + bitrev(k, bits)] = v;
-    });
-    if constexpr (LOWER_ONLY) dit_lower_only<R, i * R, 16>(x);
-    else dit<R, i * R, 16>(x);
-  });
-}
-
-template <class P, int R, int S>
-__device__ __forceinline__ void inv_store(const cf (&x)[16], int t, float2* row) {
-  constexpr int NB = 16 / R;
-  static_for<0, NB>([&](auto ii) {
-    constexpr int i = decltype(ii)::value;
-    const int q = t + P::T * i;
-    const int b = q / S, m = q % S;
-    float2* pb = row + phys(b * (S * R) + m);
-    static_for<0, R>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      lds_put(pb, poff(j * S), x[i * R + j]);
-    });
-  });
-}
-
-// twiddle bases of one pass for thread t: exp(-2 pi i m / (S R)), one per butterfly when the
-// thread's butterflies have different offsets (first pass only), else a single shared one.
-template <class P, int R, int S>
-__device__ __forceinline__ void pass_bases(int t, cf (&w)[16 / R]) {
-  constexpr int NB = 16 / R;
-  static_for<0, NB>([&](auto ii) {
-    constexpr int i = decltype(ii)::value;
-    if constexpr (S > P::T || i == 0) {
-      const int q = t + P::T * i;
-      w[i] = unit_root(q % S, S * R);
-    } else {
-      w[i] = w[0];
-    }
-  });
-}
-
-// group taken by work item w in the paired radix-8 pass, and the group with the mirrored frequencies
-template <class P>
-__device__ __forceinline__ void paired_groups(int w, int& g, int& g2) {
-  constexpr int RL = P::RL, R1 = P::R1, R2 = P::R2, R3 = P::R3;
-  g = (w / (RL / 2)) * RL + (w % (RL / 2));
-  if (w == 0) {            // groups 0 (k_low = 0) and RL/2 (k_low = M/2) are both self-mirrored
-    g2 = RL / 2;
-    return;
-  }
-  int k1 = g / (R2 * R3), k2 = (g / R3) % R2, k3 = g % R3;
-  if (k1) {
-    k1 = R1 - k1; k2 = R2 - 1 - k2; k3 = R3 - 1 - k3;
-  } else if (k2) {
-    k2 = R2 - k2; k3 = R3 - 1 - k3;
-  } else {
-    k3 = R3 - k3;
-  }
-  g2 = (k1 * R2 + k2) * R3 + k3;
-}
-
-// ------------------------------------------------------------------------------------------
-// forward FFT up to (and including) the paired radix-8 pass.  On return x[0..8) holds group g
-// and x[8..16) holds group g2, both in bit-reversed register order.
-// ------------------------------------------------------------------------------------------
-template <class P, bool ZERO_UPPER>
-__device__ __forceinline__ void forward_to_pairs(cf (&x)[16], int t, float2* row, const cf (&wb1)[16 / P::R1],
-                                                 const cf (&wb2)[16 / P::R2], const cf (&wb3)[16 / P::R3],
-                                                 int g, int g2) {
-  fwd_compute_store<P, P::R1, P::S1, ZERO_UPPER>(x, t, row, wb1);
-  __syncthreads();
-  fwd_load<P, P::R2, P::S2>(x, t, row);
-  fwd_compute_store<P, P::R2, P::S2, false>(x, t, row, wb2);
-  __syncthreads();
-  if constexpr (P::R3 > 1) {
-    fwd_load<P, P::R3, P::S3>(x, t, row);
-    fwd_compute_store<P, P::R3, P::S3, false>(x, t, row, wb3);
-    __syncthreads();
-  }
-  {
-    const float2* pa = row + phys(g * 8);
-    const float2* pb = row + phys(g2 * 8);
-    static_for<0, 8>([&](auto jj) {
-      constexpr int j = decltype(jj)::value;
-      x[j] = lds_get(pa, j);
-      x[8 + j] = lds_get(pb, j);
-    });
-  }
-  dif<8, 0, 16>(x);
-  dif<8, 8, 16>(x);
-}
-
-// One spectral pair: za sits at frequency k, zb at N-k.  Returns W[k] in za and W[N-k] in zb.
-__device__ __forceinline__ void pair_multiply(cf& za, cf& zb, float4 K) {
-  cf A = {0.5f * (za.re + zb.re), 0.5f * (za.im - zb.im)};        // (Z[k] + conj Z[N-k]) / 2
-  cf Bq = {0.5f * (za.im + zb.im), 0.5f * (zb.re - za.re)};       // (Z[k] - conj Z[N-k]) / (2i)
-  cf Pp = cmul(A, cf{K.x, K.y});
-  cf Q = cmul(Bq, cf{K.z, K.w});
-  za = {Pp.re - Q.im, Pp.im + Q.re};                               // P + iQ
-  zb = {Pp.re + Q.im, Q.re - Pp.im};                               // conj(P) + i conj(Q)
-}
 
 // ------------------------------------------------------------------------------------------
 // K2: the fused mixer core
@@ -422,27 +225,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
     }
 
     // ---- inverse ----
-    dit<8, 0, 16>(x);
-    dit<8, 8, 16>(x);
-    {
-      float2* pa = row + phys(g * 8);
-      float2* pb = row + phys(g2 * 8);
-      static_for<0, 8>([&](auto jj) {
-        constexpr int j = decltype(jj)::value;
-        lds_put(pa, j, x[j]);
-        lds_put(pb, j, x[8 + j]);
-      });
-    }
-    __syncthreads();
-    if constexpr (P::R3 > 1) {
-      inv_load_compute<P, P::R3, P::S3, false>(x, t, row, wb3);
-      inv_store<P, P::R3, P::S3>(x, t, row);
-      __syncthreads();
-    }
-    inv_load_compute<P, P::R2, P::S2, false>(x, t, row, wb2);
-    inv_store<P, P::R2, P::S2>(x, t, row);
-    __syncthreads();
-    inv_load_compute<P, P::R1, P::S1, true>(x, t, row, wb1);
+    inverse_from_pairs<P, true>(x, t, row, wb1, wb2, wb3, g, g2);
     inv_store_lower<P>(x, t, row);      // only slots this thread has just read are overwritten
     __syncthreads();
 
@@ -591,13 +374,20 @@ static int launch_filter_spectrum(const float* taps1, const float* taps2, const 
   X(13, 16, 8, 8)           \
   X(14, 16, 16, 8)
 
+// N = 65536 (four sub-transforms per row), defined in fftconv_big_kernels.hip
+int launch_mixer_core_big_dispatch(const void* xproj, const float* u, const float* sw, const float* sb,
+                                   const float* pbias, const float* spec, void* y, int B, int d, int act_dtype,
+                                   hipStream_t stream);
+int launch_filter_spectrum_big(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
+                               int d, hipStream_t stream);
+
 }  // namespace m2
 
 using namespace m2;
 
 extern "C" int m2_fftconv_supported_seqlen(int L) {
   int n = 2 * L;
-  return (n >= 256 && n <= 16384 && (n & (n - 1)) == 0) ? 1 : 0;
+  return (n >= 256 && n <= 65536 && n != 32768 && (n & (n - 1)) == 0) ? 1 : 0;
 }
 
 extern "C" size_t m2_filter_spectrum_bytes(int d, int L) {
@@ -609,8 +399,9 @@ extern "C" int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, co
   if (!taps1 || !spec) return set_error(M2_ERR_ARG, "m2_filter_spectrum_fwd: null pointer");
   if (d <= 0) return set_error(M2_ERR_ARG, "m2_filter_spectrum_fwd: d must be positive, got %d", d);
   if (!m2_fftconv_supported_seqlen(L))
-    return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: L=%d unsupported (need 2L a power of two in [256, 16384])", L);
+    return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: L=%d unsupported (need 2L a power of two in [256, 16384], or 65536)", L);
   const int logn = ilog2(2 * L);
+  if (logn == 16) return launch_filter_spectrum_big(taps1, taps2, D1, D2, spec, d, (hipStream_t)stream);
   switch (logn) {
 #define X(LOGN, R1, R2, R3) \
   case LOGN:                \
@@ -629,9 +420,10 @@ extern "C" int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, cons
   if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
     return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
   if (!m2_fftconv_supported_seqlen(L))
-    return set_error(M2_ERR_UNSUPPORTED, "m2_mixer_core_fwd: L=%d unsupported (need 2L a power of two in [256, 16384])", L);
+    return set_error(M2_ERR_UNSUPPORTED, "m2_mixer_core_fwd: L=%d unsupported (need 2L a power of two in [256, 16384], or 65536)", L);
   const int logn = ilog2(2 * L);
   hipStream_t s = (hipStream_t)stream;
+  if (logn == 16) return launch_mixer_core_big_dispatch(xproj, u, short_w, short_b, proj_bias, spec, y, B, d, act_dtype, s);
   switch (logn) {
 #define X(LOGN, R1, R2, R3)                                                                                       \
   case LOGN:                                                                                                      \
@@ -651,9 +443,10 @@ extern "C" int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, 
   if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
     return set_error(M2_ERR_ARG, "m2_fftconv_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
   if (!m2_fftconv_supported_seqlen(L))
-    return set_error(M2_ERR_UNSUPPORTED, "m2_fftconv_fwd: L=%d unsupported (need 2L a power of two in [256, 16384])", L);
+    return set_error(M2_ERR_UNSUPPORTED, "m2_fftconv_fwd: L=%d unsupported (need 2L a power of two in [256, 16384], or 65536)", L);
   const int logn = ilog2(2 * L);
   hipStream_t s = (hipStream_t)stream;
+  if (logn == 16) return launch_mixer_core_big_dispatch(x, nullptr, nullptr, nullptr, nullptr, spec, y, B, d, act_dtype, s);
   switch (logn) {
 #define X(LOGN, R1, R2, R3)                                                                                  \
   case LOGN:                                                                                                 \

@@ -35,6 +35,9 @@ def test_size_queries_and_argument_checks_without_gpu():
     lib = _lib.lib
     assert lib.m2_fftconv_supported_seqlen(128) == 1
     assert lib.m2_fftconv_supported_seqlen(8192) == 1
+    assert lib.m2_fftconv_supported_seqlen(32768) == 1
+    assert lib.m2_fftconv_supported_seqlen(16384) == 0
+    assert lib.m2_fftconv_supported_seqlen(65536) == 0
     assert lib.m2_fftconv_supported_seqlen(64) == 0
     assert lib.m2_fftconv_supported_seqlen(100) == 0
     assert lib.m2_filter_spectrum_bytes(768, 8192) == 768 * 8192 * 16
