@@ -30,6 +30,8 @@ struct Plan {
   static constexpr int WG = T < 256 ? 256 : T;    // threads per workgroup
   static constexpr int RPW = WG / T;              // rows per workgroup
   static constexpr int ROW_LDS = N + (N >> 4);    // padded complex slots per row
+  static constexpr int TW_LDS = R2 * (N / R1 / R2) + (R3_ > 1 ? R3_ * (N / R1 / R2 / R3_) : 0);   // twiddle tables
+  static constexpr int WG_LDS = (T < 256 ? 256 / T : 1) * ROW_LDS + TW_LDS;                         // float2 slots per workgroup
   static_assert(R1 * R2 * R3 * RP == N, "radices must multiply to N");
   static_assert(S3 == RP, "last stride");
   static_assert(R1 * R2 >= E, "passes after the first must share twiddles inside a thread");
@@ -58,9 +60,60 @@ __device__ __forceinline__ cf unit_root(int m, int n) {
 // ------------------------------------------------------------------------------------------
 // generic passes on the row held in LDS
 // ------------------------------------------------------------------------------------------
+// Twiddles.  Pass 1 twiddles w_N^(m k) are different for every thread: they are computed once per
+// kernel and stay in registers.  The twiddles of the later passes depend only on (m, k) with m below
+// the pass stride, i.e. they are the same small table for every row and every thread block of the
+// pass: tables in LDS ([k][m], conflict-free for consecutive m), built once per workgroup.
+template <class P>
+struct Twiddles {
+  cf p1[16 / P::R1][P::R1];     // [butterfly][k], k = 1 .. R1-1
+  const float2* tab2;           // [R2][S2]
+  const float2* tab3;           // [R3][S3]   (R3 > 1 only)
+  static constexpr int TAB2 = P::R2 * P::S2;
+  static constexpr int TAB3 = (P::R3 > 1) ? P::R3 * P::S3 : 0;
+  static constexpr int LDS_SLOTS = TAB2 + TAB3;       // float2 slots after the row buffers
+};
+
+// Must be called by every thread of the workgroup (it contains a barrier).
+template <class P>
+__device__ __forceinline__ void twiddles_init(Twiddles<P>& tw, int t, float2* tables) {
+  constexpr int NB = 16 / P::R1;
+  static_for<0, NB>([&](auto ii) {
+    constexpr int i = decltype(ii)::value;
+    const int q = t + P::T * i;
+    powers<P::R1>(unit_root(q % P::S1, P::S1 * P::R1), tw.p1[i]);
+  });
+  tw.tab2 = tables;
+  tw.tab3 = tables + Twiddles<P>::TAB2;
+  for (int e = threadIdx.x; e < Twiddles<P>::TAB2; e += blockDim.x) {
+    const int k = e / P::S2, m = e % P::S2;
+    const cf w = unit_root((k * m) % (P::S2 * P::R2), P::S2 * P::R2);
+    tables[e] = make_float2(w.re, w.im);
+  }
+  if constexpr (P::R3 > 1) {
+    for (int e = threadIdx.x; e < Twiddles<P>::TAB3; e += blockDim.x) {
+      const int k = e / P::S3, m = e % P::S3;
+      const cf w = unit_root((k * m) % (P::S3 * P::R3), P::S3 * P::R3);
+      tables[Twiddles<P>::TAB2 + e] = make_float2(w.re, w.im);
+    }
+  }
+  __syncthreads();
+}
+
+// twiddle w^(m k) of pass PASS (1, 2 or 3) for butterfly i of this thread
+template <class P, int PASS, int S, int I, int K>
+__device__ __forceinline__ cf pass_twiddle(const Twiddles<P>& tw, int m) {
+  if constexpr (PASS == 1) {
+    return tw.p1[I][K];
+  } else {
+    const float2 v = (PASS == 2 ? tw.tab2 : tw.tab3)[K * S + m];
+    return {v.x, v.y};
+  }
+}
+
 // forward: registers hold natural-order inputs of E/R butterflies; butterfly, twiddle, store.
-template <class P, int R, int S, bool ZERO_UPPER>
-__device__ __forceinline__ void fwd_compute_store(cf (&x)[16], int t, float2* row, const cf (&wbase)[16 / R]) {
+template <class P, int PASS, int R, int S, bool ZERO_UPPER>
+__device__ __forceinline__ void fwd_compute_store(cf (&x)[16], int t, float2* row, const Twiddles<P>& tw) {
   constexpr int NB = 16 / R;
   static_for<0, NB>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
@@ -68,14 +121,12 @@ __device__ __forceinline__ void fwd_compute_store(cf (&x)[16], int t, float2* ro
     const int b = q / S, m = q % S;
     if constexpr (ZERO_UPPER) dif_zero_upper<R, i * R, 16>(x);
     else dif<R, i * R, 16>(x);
-    cf p[R];
-    powers<R>(wbase[(S > P::T) ? i : 0], p);
     float2* pb = row + phys(b * (S * R) + m);
     constexpr int bits = ilog2(R);
     static_for<0, R>([&](auto kk) {
       constexpr int k = decltype(kk)::value;
       cf v = x[i * R + bitrev(k, bits)];
-      if constexpr (k > 0) v = cmul(v, p[k]);
+      if constexpr (k > 0) v = cmul(v, pass_twiddle<P, PASS, S, i, k>(tw, m));
       lds_put(pb, poff(k * S), v);
     });
   });
@@ -97,21 +148,19 @@ __device__ __forceinline__ void fwd_load(cf (&x)[16], int t, const float2* row) 
 }
 
 // inverse: load digit k into bit-reversed register, conj twiddle, inverse butterfly (natural out)
-template <class P, int R, int S, bool LOWER_ONLY>
-__device__ __forceinline__ void inv_load_compute(cf (&x)[16], int t, const float2* row, const cf (&wbase)[16 / R]) {
+template <class P, int PASS, int R, int S, bool LOWER_ONLY>
+__device__ __forceinline__ void inv_load_compute(cf (&x)[16], int t, const float2* row, const Twiddles<P>& tw) {
   constexpr int NB = 16 / R;
   static_for<0, NB>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
     const int q = t + P::T * i;
     const int b = q / S, m = q % S;
-    cf p[R];
-    powers<R>(wbase[(S > P::T) ? i : 0], p);
     const float2* pb = row + phys(b * (S * R) + m);
     constexpr int bits = ilog2(R);
     static_for<0, R>([&](auto kk) {
       constexpr int k = decltype(kk)::value;
       cf v = lds_get(pb, poff(k * S));
-      if constexpr (k > 0) v = cmulc(v, p[k]);
+      if constexpr (k > 0) v = cmulc(v, pass_twiddle<P, PASS, S, i, k>(tw, m));
       x[i * R + bitrev(k, bits)] = v;
     });
     if constexpr (LOWER_ONLY) dit_lower_only<R, i * R, 16>(x);
@@ -131,22 +180,6 @@ __device__ __forceinline__ void inv_store(const cf (&x)[16], int t, float2* row)
       constexpr int j = decltype(jj)::value;
       lds_put(pb, poff(j * S), x[i * R + j]);
     });
-  });
-}
-
-// twiddle bases of one pass for thread t: exp(-2 pi i m / (S R)), one per butterfly when the
-// thread's butterflies have different offsets (first pass only), else a single shared one.
-template <class P, int R, int S>
-__device__ __forceinline__ void pass_bases(int t, cf (&w)[16 / R]) {
-  constexpr int NB = 16 / R;
-  static_for<0, NB>([&](auto ii) {
-    constexpr int i = decltype(ii)::value;
-    if constexpr (S > P::T || i == 0) {
-      const int q = t + P::T * i;
-      w[i] = unit_root(q % S, S * R);
-    } else {
-      w[i] = w[0];
-    }
   });
 }
 
@@ -175,17 +208,15 @@ __device__ __forceinline__ void paired_groups(int w, int& g, int& g2) {
 // and x[8..16) holds group g2, both in bit-reversed register order.
 // ------------------------------------------------------------------------------------------
 template <class P, bool ZERO_UPPER>
-__device__ __forceinline__ void forward_to_pairs(cf (&x)[16], int t, float2* row, const cf (&wb1)[16 / P::R1],
-                                                 const cf (&wb2)[16 / P::R2], const cf (&wb3)[16 / P::R3],
-                                                 int g, int g2) {
-  fwd_compute_store<P, P::R1, P::S1, ZERO_UPPER>(x, t, row, wb1);
+__device__ __forceinline__ void forward_to_pairs(cf (&x)[16], int t, float2* row, const Twiddles<P>& tw, int g, int g2) {
+  fwd_compute_store<P, 1, P::R1, P::S1, ZERO_UPPER>(x, t, row, tw);
   __syncthreads();
   fwd_load<P, P::R2, P::S2>(x, t, row);
-  fwd_compute_store<P, P::R2, P::S2, false>(x, t, row, wb2);
+  fwd_compute_store<P, 2, P::R2, P::S2, false>(x, t, row, tw);
   __syncthreads();
   if constexpr (P::R3 > 1) {
     fwd_load<P, P::R3, P::S3>(x, t, row);
-    fwd_compute_store<P, P::R3, P::S3, false>(x, t, row, wb3);
+    fwd_compute_store<P, 3, P::R3, P::S3, false>(x, t, row, tw);
     __syncthreads();
   }
   {
@@ -215,9 +246,8 @@ __device__ __forceinline__ void pair_multiply(cf& za, cf& zb, float4 K) {
 // Inverse of forward_to_pairs: x[0..8) / x[8..16) hold groups g / g2 in bit-reversed register order.
 // On return x[i R1 + j] is the (unscaled) time sample n = t + T i + j S1; with LOWER_ONLY only j < R1/2.
 template <class P, bool LOWER_ONLY>
-__device__ __forceinline__ void inverse_from_pairs(cf (&x)[16], int t, float2* row, const cf (&wb1)[16 / P::R1],
-                                                   const cf (&wb2)[16 / P::R2], const cf (&wb3)[16 / P::R3],
-                                                   int g, int g2) {
+__device__ __forceinline__ void inverse_from_pairs(cf (&x)[16], int t, float2* row, const Twiddles<P>& tw, int g,
+                                                   int g2) {
   dit<8, 0, 16>(x);
   dit<8, 8, 16>(x);
   {
@@ -231,14 +261,14 @@ __device__ __forceinline__ void inverse_from_pairs(cf (&x)[16], int t, float2* r
   }
   __syncthreads();
   if constexpr (P::R3 > 1) {
-    inv_load_compute<P, P::R3, P::S3, false>(x, t, row, wb3);
+    inv_load_compute<P, 3, P::R3, P::S3, false>(x, t, row, tw);
     inv_store<P, P::R3, P::S3>(x, t, row);
     __syncthreads();
   }
-  inv_load_compute<P, P::R2, P::S2, false>(x, t, row, wb2);
+  inv_load_compute<P, 2, P::R2, P::S2, false>(x, t, row, tw);
   inv_store<P, P::R2, P::S2>(x, t, row);
   __syncthreads();
-  inv_load_compute<P, P::R1, P::S1, LOWER_ONLY>(x, t, row, wb1);
+  inv_load_compute<P, 1, P::R1, P::S1, LOWER_ONLY>(x, t, row, tw);
 }
 
 }  // namespace m2

@@ -160,10 +160,6 @@ __device__ __forceinline__ void stage_sub_input(int k1, int t, float2* row, LOAD
   }
 }
 
-struct BigTwiddles {
-  cf wb1[1], wb2[1], wb3[2];
-};
-
 template <typename ACT>
 __global__ __launch_bounds__(1024) void mixer_core_big_kernel(
     const ACT* __restrict__ xproj, const float* __restrict__ uin, const float* __restrict__ sw,
@@ -174,10 +170,8 @@ __global__ __launch_bounds__(1024) void mixer_core_big_kernel(
   extern __shared__ float2 lds[];
   float2* row = lds;
   const int t = threadIdx.x;
-  cf wb1[16 / P::R1], wb2[16 / P::R2], wb3[16 / P::R3];
-  pass_bases<P, P::R1, P::S1>(t, wb1);
-  pass_bases<P, P::R2, P::S2>(t, wb2);
-  pass_bases<P, P::R3, P::S3>(t, wb3);
+  Twiddles<P> tw;
+  twiddles_init<P>(tw, t, lds + P::RPW * P::ROW_LDS);
   int g, gm;
   paired_groups<P>(t, g, gm);
   const int gc = complement_group<P>(g);
@@ -219,11 +213,11 @@ __global__ __launch_bounds__(1024) void mixer_core_big_kernel(
       stage_sub_input<2>(k1, t, row, loadz);
       __syncthreads();
       fwd_load<P, P::R1, P::S1>(x, t, row);
-      forward_to_pairs<P, false>(x, t, row, wb1, wb2, wb3, g, gsel);
+      forward_to_pairs<P, false>(x, t, row, tw, g, gsel);
     };
     // inverse sub-transform k1 from x, accumulate into the two output halves
     auto inverse = [&](int k1, int gsel, cf (&x)[16]) __attribute__((always_inline)) {
-      inverse_from_pairs<P, false>(x, t, row, wb1, wb2, wb3, g, gsel);
+      inverse_from_pairs<P, false>(x, t, row, tw, g, gsel);
       __syncthreads();            // the next stage overwrites LDS that this pass has just read
       // conj(w_N^(k1 (t + 1024 j))) = conj(w_N^(k1 t)) conj(w_64^(k1 j))
       const cf base = unit_root((k1 * t) & (kBigN - 1), kBigN);
@@ -324,10 +318,8 @@ __global__ __launch_bounds__(1024) void filter_spectrum_big_kernel(
   extern __shared__ float2 lds[];
   float2* row = lds;
   const int t = threadIdx.x;
-  cf wb1[16 / P::R1], wb2[16 / P::R2], wb3[16 / P::R3];
-  pass_bases<P, P::R1, P::S1>(t, wb1);
-  pass_bases<P, P::R2, P::S2>(t, wb2);
-  pass_bases<P, P::R3, P::S3>(t, wb3);
+  Twiddles<P> tw;
+  twiddles_init<P>(tw, t, lds + P::RPW * P::ROW_LDS);
   int g, gm;
   paired_groups<P>(t, g, gm);
   const int gc = complement_group<P>(g);
@@ -349,7 +341,7 @@ __global__ __launch_bounds__(1024) void filter_spectrum_big_kernel(
       stage_sub_input<4>(k1, t, row, loadz);
       __syncthreads();
       fwd_load<P, P::R1, P::S1>(x, t, row);
-      forward_to_pairs<P, false>(x, t, row, wb1, wb2, wb3, g, gsel);
+      forward_to_pairs<P, false>(x, t, row, tw, g, gsel);
       __syncthreads();            // LDS is reused by the next sub-transform
     };
     auto split = [&](cf za, cf zb) -> float4 {
@@ -395,7 +387,7 @@ __global__ __launch_bounds__(1024) void filter_spectrum_big_kernel(
 template <typename ACT>
 int launch_mixer_core_big(const void* xproj, const float* u, const float* sw, const float* sb, const float* pbias,
                           const float* spec, void* y, int B, int d, hipStream_t stream) {
-  const size_t lds_bytes = (size_t)BigPlan::ROW_LDS * sizeof(float2);
+  const size_t lds_bytes = (size_t)BigPlan::WG_LDS * sizeof(float2);
   auto kern = mixer_core_big_kernel<ACT>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(mixer_core_big): %s", hipGetErrorString(e));
@@ -416,7 +408,7 @@ int launch_mixer_core_big_dispatch(const void* xproj, const float* u, const floa
 
 int launch_filter_spectrum_big(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
                                int d, hipStream_t stream) {
-  const size_t lds_bytes = (size_t)BigPlan::ROW_LDS * sizeof(float2);
+  const size_t lds_bytes = (size_t)BigPlan::WG_LDS * sizeof(float2);
   hipError_t e = hipFuncSetAttribute((const void*)filter_spectrum_big_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds_bytes);
   if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(filter_spectrum_big): %s", hipGetErrorString(e));

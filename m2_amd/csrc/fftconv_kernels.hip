@@ -123,10 +123,8 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
   float2* row = lds + rloc * P::ROW_LDS;
   const int n0 = 8 * t;
 
-  cf wb1[16 / P::R1], wb2[16 / P::R2], wb3[16 / P::R3];
-  pass_bases<P, P::R1, P::S1>(t, wb1);
-  pass_bases<P, P::R2, P::S2>(t, wb2);
-  if constexpr (P::R3 > 1) pass_bases<P, P::R3, P::S3>(t, wb3);
+  Twiddles<P> tw;
+  twiddles_init<P>(tw, t, lds + P::RPW * P::ROW_LDS);
   int g, g2;
   paired_groups<P>(t, g, g2);
 
@@ -196,7 +194,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
 
     cf x[16];
     fwd_load_lower<P>(x, t, row);
-    forward_to_pairs<P, true>(x, t, row, wb1, wb2, wb3, g, g2);
+    forward_to_pairs<P, true>(x, t, row, tw, g, g2);
 
     // ---- spectral multiply in registers ----
     {
@@ -225,7 +223,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
     }
 
     // ---- inverse ----
-    inverse_from_pairs<P, true>(x, t, row, wb1, wb2, wb3, g, g2);
+    inverse_from_pairs<P, true>(x, t, row, tw, g, g2);
     inv_store_lower<P>(x, t, row);      // only slots this thread has just read are overwritten
     __syncthreads();
 
@@ -262,10 +260,8 @@ __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
   float2* row = lds + rloc * P::ROW_LDS;
   const int n0 = 16 * t;
 
-  cf wb1[16 / P::R1], wb2[16 / P::R2], wb3[16 / P::R3];
-  pass_bases<P, P::R1, P::S1>(t, wb1);
-  pass_bases<P, P::R2, P::S2>(t, wb2);
-  if constexpr (P::R3 > 1) pass_bases<P, P::R3, P::S3>(t, wb3);
+  Twiddles<P> tw;
+  twiddles_init<P>(tw, t, lds + P::RPW * P::ROW_LDS);
   int g, g2;
   paired_groups<P>(t, g, g2);
   const float scale = 0.5f / (float)N;       // the 1/2 of the even/odd split and the 1/N of the convolution
@@ -293,7 +289,7 @@ __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
     __syncthreads();
     cf x[16];
     fwd_load<P, P::R1, P::S1>(x, t, row);
-    forward_to_pairs<P, false>(x, t, row, wb1, wb2, wb3, g, g2);
+    forward_to_pairs<P, false>(x, t, row, tw, g, g2);
     __syncthreads();      // LDS is reused by the next row
 
     float4 K[8];
@@ -332,7 +328,7 @@ __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
 template <class P, typename ACT>
 static int launch_mixer_core(const void* xproj, const float* u, const float* sw, const float* sb, const float* pbias,
                              const float* spec, void* y, int B, int d, hipStream_t stream) {
-  const size_t lds_bytes = (size_t)P::RPW * P::ROW_LDS * sizeof(float2);
+  const size_t lds_bytes = (size_t)P::WG_LDS * sizeof(float2);
   auto kern = mixer_core_kernel<P, ACT>;
   if (lds_bytes > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -352,7 +348,7 @@ static int launch_mixer_core(const void* xproj, const float* u, const float* sw,
 template <class P>
 static int launch_filter_spectrum(const float* taps1, const float* taps2, const float* D1, const float* D2,
                                   float* spec, int d, hipStream_t stream) {
-  const size_t lds_bytes = (size_t)P::RPW * P::ROW_LDS * sizeof(float2);
+  const size_t lds_bytes = (size_t)P::WG_LDS * sizeof(float2);
   auto kern = filter_spectrum_kernel<P>;
   if (lds_bytes > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
