@@ -27,6 +27,10 @@ import time
 import torch
 
 HBM_PEAK_GBPS = 8000.0
+# HBM-side bytes per mixer-core launch at the default workload, from the two rocprofv3 --pmc runs
+# (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000 against a plain 256 MiB copy); summary in
+# profiles/mixer_core_L8192_B4_hbm_traffic.md.  Only valid for --config c3.
+MIXER_CORE_TRAFFIC_BYTES_C3 = int((344848 * 2.0 + 78848 * 1.0) * 1024)
 
 
 def workload(name: str):
@@ -122,11 +126,24 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 256 MiB device copy three times (known-size kernel for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
+
+    if args.calibrate_copy:
+        n = 256 * 1024 * 1024 // 4
+        src = torch.zeros(n, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": n * 4, "calibrate_copy_bytes_written": n * 4, "repeats": 3}))
+        return
 
     import m2_amd
     from m2_amd import ops
@@ -181,7 +198,8 @@ def main():
                    "filters": "regenerated from weights every forward"},
         "roofline": {"kernel": "mixer_core_kernel (short conv + gates + two FFT long convs + add)",
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": MIXER_CORE_TRAFFIC_BYTES_C3 if args.config == "c3" else None,
                      "bytes_per_launch": nbytes, "ms_per_launch": t_core, "launches_timed": timer.count("mixer_core"),
                      "achieved_incl_filter_generation": nbytes / ((t_core + t_filt) * 1e-3) / 1e9,
                      "filter_generation_ms_per_layer": t_filt},
