@@ -68,7 +68,7 @@ size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int order);
  *                                      taps[f][c][L + l]  = k_rev[c][L-1-l]   (0 if not bidirectional)
  * with k[c][l] = (W3 sin(f.(W2 sin(f.(W1 sin(f.(W0 z_l + b0)) + b1)) + b2)))[c] * (exp(-t_l |delta_c|) + shift),
  * f = w_mod * freq.  `params` is a HOST array of nfilters structs holding DEVICE pointers.
- * Supported: order == 128, 3 <= emb_dim <= 8, d % 64 == 0, L % 64 == 0. */
+ * Supported: order == 128, 3 <= emb_dim <= 8, d % 64 == 0, L % 32 == 0. */
 int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order, int emb_dim,
                         float w_mod, float shift, float* workspace, float* taps, void* stream);
 

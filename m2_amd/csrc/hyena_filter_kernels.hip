@@ -6,9 +6,13 @@
 // (bert/src/mm/hyena_utils.py:168-175 the MLP, :50-63 Sin, :110-112 modulation, :201-217 filter /
 // filter_rev, :231-236 placement of the forward and the flipped reverse taps in a 2L window.)
 //
-// Two kernels.  `hidden_kernel` evaluates the three sin layers for a tile of positions with the
-// activations resident in LDS and writes h3 (L, 128) per MLP.  `project_kernel` is the 128 -> d
-// projection as an fp32 MFMA GEMM (v_mfma_f32_32x32x2_f32) whose epilogue applies the decay and
+// Two kernels.  `hidden_kernel` evaluates the three sin layers for a tile of 32 positions: the first
+// (emb -> 128) on the vector ALU, the two 128 x 128 layers as fp32 MFMA GEMMs
+// (v_mfma_f32_32x32x2_f32: exact fp32 products, which matters because sin(freq * x) amplifies any
+// rounding of x) with the activations resident in LDS; it writes h3 split into a bf16 high part and
+// a bf16 low part (h3 = hi + lo to 16 mantissa bits).  `project_kernel` is the 128 -> d projection as
+// a three-product split-bf16 MFMA GEMM (W_hi h_hi + W_hi h_lo + W_lo h_hi, v_mfma_f32_32x32x16_bf16,
+// fp32 accumulate; 4.6e-6 relative error against fp64, measured) whose epilogue applies the decay and
 // stores the taps channel-major, forward taps at [0, L) and reverse taps mirrored into [L, 2L).
 #include <hip/hip_runtime.h>
 
@@ -32,24 +36,31 @@ struct FilterBatch {
   FilterPtrs f[kMaxFilters];
 };
 
-// grid (L / kPosTile, 2 * nfilters), block 128: thread o owns output neuron o.
-__global__ __launch_bounds__(kOrder) void hidden_kernel(FilterBatch fb, int L, int emb, float w_mod,
-                                                        float* __restrict__ hidden /* (2 nf, L, 128) */) {
-  __shared__ float act[2][kPosTile][kOrder];
-  const int o = threadIdx.x;
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kActRow = kOrder + 4;       // padded fp32 row of the activation tile (bank-conflict-free b128 reads)
+
+// grid (L / 32, 2 * nfilters), block 256 = 4 waves; wave w owns output neurons [32 w, 32 w + 32).
+__global__ __launch_bounds__(256) void hidden_kernel(FilterBatch fb, int L, int emb, float w_mod,
+                                                     uint16_t* __restrict__ h_hi /* (2 nf, L, 128) bf16 */,
+                                                     uint16_t* __restrict__ h_lo /* (2 nf, L, 128) bf16 */) {
+  __shared__ __attribute__((aligned(16))) float act[2][kPosTile][kActRow];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
   const int fi = blockIdx.y >> 1, dir = blockIdx.y & 1;
   const FilterPtrs& F = fb.f[fi];
   const MlpPtrs& W = F.mlp[dir];
   if (W.w0 == nullptr) return;                  // not bidirectional: nothing to do for dir == 1
   const int l0 = blockIdx.x * kPosTile;
-  const float fo = w_mod * F.freq[o];
 
-  // layer 0: emb -> 128
+  // layer 0 (emb -> 128) on the vector ALU: thread = (neuron o, 16 positions)
   {
+    const int o = tid & (kOrder - 1), p0 = (tid >> 7) * 16;
     float w[kMaxEmb];
     for (int e = 0; e < kMaxEmb; ++e) w[e] = e < emb ? W.w0[o * emb + e] : 0.f;
-    const float b = W.b0[o];
-    for (int p = 0; p < kPosTile; ++p) {
+    const float b = W.b0[o], fo = w_mod * F.freq[o];
+    for (int p = p0; p < p0 + 16; ++p) {
       const float* zp = F.z + (long)(l0 + p) * emb;
       float acc = b;
       for (int e = 0; e < emb; ++e) acc += w[e] * zp[e];
@@ -57,79 +68,133 @@ __global__ __launch_bounds__(kOrder) void hidden_kernel(FilterBatch fb, int L, i
     }
   }
   __syncthreads();
-  // layers 1, 2: 128 -> 128 with the weight row in registers and activations broadcast from LDS
+  // layers 1, 2: D[o'][pos] = sum_o W[o'][o] act[pos][o].  Lane (i32, half) holds K = 8 q + 4 half + {0..3}
+  // of weight row 32 wave + i32 and of position i32: four MFMA steps per pair of float4.
   for (int layer = 0; layer < 2; ++layer) {
-    const float* wrow = (layer == 0 ? W.w1 : W.w2) + (long)o * kOrder;
-    const float b = (layer == 0 ? W.b1 : W.b2)[o];
-    float4 w[kOrder / 4];
-#pragma unroll
-    for (int i = 0; i < kOrder / 4; ++i) w[i] = reinterpret_cast<const float4*>(wrow)[i];
+    const float* wm = (layer == 0 ? W.w1 : W.w2) + (long)(32 * wave + i32) * kOrder + 4 * half;
+    const float* bias = layer == 0 ? W.b1 : W.b2;
     const int src = layer & 1, dst = src ^ 1;
-    for (int p = 0; p < kPosTile; ++p) {
-      const float4* a = reinterpret_cast<const float4*>(act[src][p]);
-      float acc0 = b, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+    float4 av[kOrder / 8];
 #pragma unroll
-      for (int i = 0; i < kOrder / 4; ++i) {
-        const float4 v = a[i];
-        acc0 += w[i].x * v.x;
-        acc1 += w[i].y * v.y;
-        acc2 += w[i].z * v.z;
-        acc3 += w[i].w * v.w;
+    for (int q = 0; q < kOrder / 8; ++q) av[q] = *reinterpret_cast<const float4*>(wm + 8 * q);
+    const float* bp = &act[src][i32][4 * half];
+    floatx16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+    for (int q = 0; q < kOrder / 8; ++q) {
+      const float4 bv = *reinterpret_cast<const float4*>(bp + 8 * q);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].x, bv.x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].y, bv.y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].z, bv.z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].w, bv.w, acc, 0, 0, 0);
+    }
+    // accumulator element v: neuron 32 wave + 8 (v / 4) + 4 half + v % 4, position i32
+    const long hrow = ((long)blockIdx.y * L + l0 + i32) * kOrder;
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq) {
+      const int o = 32 * wave + 8 * vq + 4 * half;
+      float s[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[j] = sinf(w_mod * F.freq[o + j] * (acc[4 * vq + j] + bias[o + j]));
+      if (layer == 0) {
+        *reinterpret_cast<float4*>(&act[dst][i32][o]) = make_float4(s[0], s[1], s[2], s[3]);
+      } else {
+        float hi[4], lo[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          hi[j] = bf16_to_f32(f32_to_bf16(s[j]));
+          lo[j] = s[j] - hi[j];
+        }
+        *reinterpret_cast<uint2*>(h_hi + hrow + o) = make_uint2(pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3]));
+        *reinterpret_cast<uint2*>(h_lo + hrow + o) = make_uint2(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]));
       }
-      const float s = sinf(fo * ((acc0 + acc1) + (acc2 + acc3)));
-      if (layer == 0) act[dst][p][o] = s;
-      else hidden[((long)blockIdx.y * L + l0 + p) * kOrder + o] = s;
     }
     __syncthreads();
   }
 }
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  u32x4 v = {a, b, c, d};
+  return __builtin_bit_cast(bf16x8, v);
+}
 
-// One wave computes a 64 (channels) x 64 (positions) tile of W3 (d x 128) * H^T (128 x L).
-// grid (L / 64, d / 64, 2 * nfilters), block 64.
-__global__ __launch_bounds__(64) void project_kernel(FilterBatch fb, int L, int d, float shift,
-                                                     const float* __restrict__ hidden /* (2 nf, L, 128) */,
-                                                     float* __restrict__ taps /* (nf, d, 2L) */) {
+// Workgroup = 4 waves; wave w owns channels [c0 + 64 w, +64) with its weight rows split into bf16
+// hi / lo parts held in registers, and walks kPosPerWg positions in tiles of 32.
+// grid (L / kPosPerWg, d / 256 rounded up, 2 * nfilters).
+constexpr int kPosPerWg = 256;      // at most; 32-position tiles past L are skipped
+__global__ __launch_bounds__(256) void project_kernel(FilterBatch fb, int L, int d, float shift,
+                                                      const uint16_t* __restrict__ h_hi, const uint16_t* __restrict__ h_lo,
+                                                      float* __restrict__ taps /* (nf, d, 2L) */) {
   const int fi = blockIdx.z >> 1, dir = blockIdx.z & 1;
   const FilterPtrs& F = fb.f[fi];
-  const int lane = threadIdx.x, i32 = lane & 31, half = lane >> 5;
-  const int c0 = blockIdx.y * 64, l0 = blockIdx.x * 64;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
+  const int c0 = blockIdx.y * 256 + wave * 64;
+  if (c0 >= d) return;
+  const int lbase = blockIdx.x * kPosPerWg;
   float* out = taps + (long)fi * d * 2 * L;
   if (F.mlp[dir].w3 == nullptr) {
     // not bidirectional: the reverse half of the window is zero
-    for (int r = 0; r < 64; ++r) out[(long)(c0 + r) * 2 * L + L + l0 + lane] = 0.f;
+    for (int r = 0; r < 64; ++r)
+      for (int p = lane; p < kPosPerWg && lbase + p < L; p += 64) out[(long)(c0 + r) * 2 * L + L + lbase + p] = 0.f;
     return;
   }
-  const float* A = F.mlp[dir].w3;                              // (d, 128), K contiguous
-  const float* Bm = hidden + (long)blockIdx.z * L * kOrder;    // (L, 128), K contiguous
-  floatx16 acc[2][2];
-  for (int a = 0; a < 2; ++a)
-    for (int b = 0; b < 2; ++b)
-      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
-  // lane (i32, half) holds K = 8q + 4 half + {0..3} of row i32: four MFMA steps per float4
-  for (int q = 0; q < kOrder / 8; ++q) {
-    float4 av[2], bv[2];
-    for (int a = 0; a < 2; ++a) av[a] = *reinterpret_cast<const float4*>(A + (long)(c0 + 32 * a + i32) * kOrder + 8 * q + 4 * half);
-    for (int b = 0; b < 2; ++b) bv[b] = *reinterpret_cast<const float4*>(Bm + (long)(l0 + 32 * b + i32) * kOrder + 8 * q + 4 * half);
-    for (int a = 0; a < 2; ++a)
-      for (int b = 0; b < 2; ++b) {
-        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[a].x, bv[b].x, acc[a][b], 0, 0, 0);
-        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[a].y, bv[b].y, acc[a][b], 0, 0, 0);
-        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[a].z, bv[b].z, acc[a][b], 0, 0, 0);
-        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[a].w, bv[b].w, acc[a][b], 0, 0, 0);
+  // A operand: rows c0 + 32 a + i32, K = 16 ks + 8 half + {0..7}, split hi / lo
+  bf16x8 ahi[2][kOrder / 16], alo[2][kOrder / 16];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    const float* wr = F.mlp[dir].w3 + (long)(c0 + 32 * a + i32) * kOrder + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < kOrder / 16; ++ks) {
+      const float4 v0 = *reinterpret_cast<const float4*>(wr + 16 * ks);
+      const float4 v1 = *reinterpret_cast<const float4*>(wr + 16 * ks + 4);
+      const float x[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+      float h[8], l[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        h[j] = bf16_to_f32(f32_to_bf16(x[j]));
+        l[j] = x[j] - h[j];
       }
+      ahi[a][ks] = as_bf16x8(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]), pack_bf16x2(h[4], h[5]), pack_bf16x2(h[6], h[7]));
+      alo[a][ks] = as_bf16x8(pack_bf16x2(l[0], l[1]), pack_bf16x2(l[2], l[3]), pack_bf16x2(l[4], l[5]), pack_bf16x2(l[6], l[7]));
+    }
   }
-  // accumulator element v of lane: row (channel) = 8 (v / 4) + 4 half + v % 4, column (position) = i32
-  for (int b = 0; b < 2; ++b) {
-    const int l = l0 + 32 * b + i32;
+  float adelta[2][16];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) adelta[a][v] = -fabsf(F.deltas[c0 + 32 * a + 8 * (v >> 2) + 4 * half + (v & 3)]) * 1.44269504088896341f;
+
+  const uint16_t* bh = h_hi + ((long)blockIdx.z * L + lbase + i32) * kOrder + 8 * half;
+  const uint16_t* bl = h_lo + ((long)blockIdx.z * L + lbase + i32) * kOrder + 8 * half;
+  for (int pt = 0; pt < kPosPerWg / 32 && lbase + pt * 32 < L; ++pt) {
+    floatx16 acc[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][v] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < kOrder / 16; ++ks) {
+      const bf16x8 bhi = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(bh + (long)pt * 32 * kOrder + 16 * ks));
+      const bf16x8 blo = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(bl + (long)pt * 32 * kOrder + 16 * ks));
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[a][ks], bhi, acc[a], 0, 0, 0);
+        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[a][ks], blo, acc[a], 0, 0, 0);
+        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[a][ks], bhi, acc[a], 0, 0, 0);
+      }
+    }
+    // accumulator element v of lane: channel c0 + 32 a + 8 (v / 4) + 4 half + v % 4, position i32
+    const int l = lbase + pt * 32 + i32;
     const float tl = F.t[l];
     const long pos = dir == 0 ? l : (2L * L - 1 - l);
+#pragma unroll
     for (int a = 0; a < 2; ++a)
+#pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int c = c0 + 32 * a + 8 * (v >> 2) + 4 * half + (v & 3);
-        const float decay = expf(-tl * fabsf(F.deltas[c])) + shift;
-        out[(long)c * 2 * L + pos] = acc[a][b][v] * decay;
+        const float decay = exp2f(tl * adelta[a][v]) + shift;        // exp(-t |delta|)
+        out[(long)c * 2 * L + pos] = acc[a][v] * decay;
       }
   }
 }
@@ -152,7 +217,8 @@ extern "C" int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfi
   if (order != kOrder) return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: order=%d, only 128 is built", order);
   if (emb_dim < 3 || emb_dim > kMaxEmb)
     return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: emb_dim=%d not in [3, %d]", emb_dim, kMaxEmb);
-  if (L <= 0 || L % 64 != 0) return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: L=%d must be a positive multiple of 64", L);
+  if (L <= 0 || L % kPosTile != 0)
+    return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: L=%d must be a positive multiple of %d", L, kPosTile);
   if (d <= 0 || d % 64 != 0) return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: d=%d must be a positive multiple of 64", d);
   FilterBatch fb;
   for (int f = 0; f < kMaxFilters; ++f) {
@@ -168,9 +234,12 @@ extern "C" int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfi
                          : MlpPtrs{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
   }
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(hidden_kernel, dim3(L / kPosTile, 2 * nfilters), dim3(kOrder), 0, s, fb, L, emb_dim, w_mod, workspace);
+  uint16_t* h_hi = reinterpret_cast<uint16_t*>(workspace);
+  uint16_t* h_lo = h_hi + (size_t)2 * nfilters * L * order;
+  hipLaunchKernelGGL(hidden_kernel, dim3(L / kPosTile, 2 * nfilters), dim3(256), 0, s, fb, L, emb_dim, w_mod, h_hi, h_lo);
   int rc = check_launch("hyena hidden_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL(project_kernel, dim3(L / 64, d / 64, 2 * nfilters), dim3(64), 0, s, fb, L, d, shift, workspace, taps);
+  hipLaunchKernelGGL(project_kernel, dim3((L + kPosPerWg - 1) / kPosPerWg, (d + 255) / 256, 2 * nfilters), dim3(256), 0, s, fb, L, d, shift,
+                     h_hi, h_lo, taps);
   return check_launch("hyena project_kernel");
 }
