@@ -147,11 +147,68 @@ class BertLayer(nn.Module):
 
 
 class BertEncoder(nn.Module):
-    def __init__(self, config: M2BertConfig):
+    """`use_hip_graph=True` captures the whole stack of layers into one HIP graph per input shape and replays
+    it: at short sequence lengths the forward is launch-bound (about ten small kernels per layer) and the
+    replay removes the per-launch host cost.  The graph holds device pointers of the weights (and of their
+    cached bf16 copies): it is dropped by `load_state_dict`, `.to()` / `.cuda()` and `reset_graphs()`; call
+    `reset_graphs()` after changing a parameter in place.  Nothing in the captured region uses a memset."""
+
+    def __init__(self, config: M2BertConfig, use_hip_graph: bool = False):
         super().__init__()
         self.layer = nn.ModuleList([BertLayer(config) for _ in range(config.num_hidden_layers)])
         self.monarch_mixer_sequence_mixing = config.monarch_mixer_sequence_mixing
         self.num_attention_heads = config.num_attention_heads
+        self.use_hip_graph = use_hip_graph
+        self._graphs = {}
+
+    # -- graph bookkeeping -------------------------------------------------------------------
+    def reset_graphs(self) -> None:
+        self._graphs = {}
+
+    def _apply(self, fn, *args, **kwargs):
+        self._graphs = {}
+        return super()._apply(fn, *args, **kwargs)
+
+    def load_state_dict(self, *args, **kwargs):
+        self._graphs = {}
+        return super().load_state_dict(*args, **kwargs)
+
+    # -- the fused schedule --------------------------------------------------------------------
+    def _run_layers(self, h32: torch.Tensor, B: int, L: int, all_layers: bool) -> List[torch.Tensor]:
+        """h32 (M, d) fp32 contiguous -> list of (M, d) fp32: every layer's output, or only the last."""
+        with torch.autocast("cuda", enabled=False):
+            h16 = h32.to(torch.bfloat16)
+            hT = h32.t().contiguous()
+            outs = []
+            n = len(self.layer)
+            o32 = h32
+            for i, layer in enumerate(self.layer):
+                want = all_layers or i == n - 1
+                o32, h16, hT = layer.fused(h16, hT, B, L, want_f32=want)
+                if want:
+                    outs.append(o32)
+        return outs
+
+    def _run_graphed(self, h32: torch.Tensor, B: int, L: int, all_layers: bool) -> List[torch.Tensor]:
+        key = (B, L, h32.shape[1], all_layers, h32.device)
+        entry = self._graphs.get(key)
+        if entry is None:
+            static_in = torch.empty_like(h32)
+            static_in.copy_(h32)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):                  # warm-up outside the capture (allocator, lazy inits)
+                self._run_layers(static_in, B, L, all_layers)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_out = self._run_layers(static_in, B, L, all_layers)
+            entry = (graph, static_in, static_out)
+            self._graphs[key] = entry
+        graph, static_in, static_out = entry
+        static_in.copy_(h32)
+        graph.replay()
+        return [o.clone() for o in static_out]
 
     def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 output_all_encoded_layers: Optional[bool] = True, subset_mask: Optional[torch.Tensor] = None,
@@ -165,36 +222,23 @@ class BertEncoder(nn.Module):
         B, L, d = hidden_states.shape
         M = B * L
         h32 = hidden_states.reshape(M, d).float().contiguous()
-        with torch.autocast("cuda", enabled=False):
-            h16 = h32.to(torch.bfloat16)
-            hT = h32.t().contiguous()
-            outs = []
-            n = len(self.layer)
-            for i, layer in enumerate(self.layer):
-                want = output_all_encoded_layers or i == n - 1
-                o32, h16, hT = layer.fused(h16, hT, B, L, want_f32=want)
-                if output_all_encoded_layers:
-                    outs.append(o32.view(B, L, d))
-            last = o32.view(B, L, d)
+        run = self._run_graphed if self.use_hip_graph else self._run_layers
+        outs = [o.view(B, L, d) for o in run(h32, B, L, bool(output_all_encoded_layers))]
         if subset_mask is not None:
-            last = last[subset_mask]
-            if output_all_encoded_layers:
-                outs[-1] = last
-        if not output_all_encoded_layers:
-            outs.append(last)
+            outs[-1] = outs[-1][subset_mask]
         return outs
 
 
 class BertModel(nn.Module):
     """Embeddings + encoder (no pooler: the heads are outside the accelerated path)."""
 
-    def __init__(self, config: M2BertConfig, add_pooling_layer: bool = False):
+    def __init__(self, config: M2BertConfig, add_pooling_layer: bool = False, use_hip_graph: bool = False):
         super().__init__()
         if add_pooling_layer:
             raise NotImplementedError("pooler / heads are not part of this path")
         self.config = config
         self.embeddings = BertEmbeddings(config)
-        self.encoder = BertEncoder(config)
+        self.encoder = BertEncoder(config, use_hip_graph=use_hip_graph)
         self.pooler = None
 
     def get_input_embeddings(self):

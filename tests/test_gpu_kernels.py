@@ -180,3 +180,37 @@ def test_encoder_small(gpu, L, B, layers):
         x = layer(x)
     e, e2 = rel_err(x, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
+
+
+def test_encoder_hip_graph_replays_match_eager(gpu):
+    """The captured encoder graph is replayed several times, with eager work and synchronisations in
+    between and with new inputs, and every replay must equal the eager result bit for bit."""
+    import m2_amd
+    cfg = m2_amd.m2_bert_80m(128)
+    cfg.num_hidden_layers = 3
+    sd = m2_amd.seeded_state_dict(cfg, 41)
+    eager = m2_amd.BertModel(cfg)
+    eager.load_state_dict(sd)
+    eager = eager.to(gpu).eval()
+    graphed = m2_amd.BertModel(cfg, use_hip_graph=True)
+    graphed.load_state_dict(sd)
+    graphed = graphed.to(gpu).eval()
+    gen = torch.Generator().manual_seed(9)
+    for it in range(5):
+        ids = torch.randint(0, cfg.vocab_size, (4, 128), generator=gen).to(gpu)
+        want, _ = eager(ids)
+        torch.cuda.synchronize()
+        scratch = torch.randn(1024, 1024, device=gpu) @ torch.randn(1024, 1024, device=gpu)     # unrelated eager work
+        got, _ = graphed(ids)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), (it, (got - want).abs().max().item())
+        del scratch
+    # all layers, second shape -> second graph
+    ids = torch.randint(0, cfg.vocab_size, (2, 128), generator=gen).to(gpu)
+    want, _ = eager(ids, output_all_encoded_layers=True)
+    for _ in range(2):
+        got, _ = graphed(ids, output_all_encoded_layers=True)
+        assert len(got) == 3 and all(torch.equal(a, b) for a, b in zip(got, want))
+    assert len(graphed.encoder._graphs) == 2
+    graphed.encoder.reset_graphs()
+    assert len(graphed.encoder._graphs) == 0
