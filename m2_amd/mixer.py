@@ -54,6 +54,8 @@ class MonarchMixerSequenceMixing(nn.Module):
         self.short_filter = nn.Conv1d(in_channels=total_width, out_channels=total_width, kernel_size=3,
                                       groups=total_width, padding=2)
         self._cast_cache = {}
+        self.cache_filters = False
+        self._spec_cache = None
 
     # -- helpers -----------------------------------------------------------------------------
     def _cast(self, name: str, p: torch.Tensor, dtype) -> torch.Tensor:
@@ -67,8 +69,25 @@ class MonarchMixerSequenceMixing(nn.Module):
         return hit[1]
 
     def filter_spectrum(self, L: int) -> torch.Tensor:
-        """Spectra of filter_fn (and filter_fn2) for sequence length L, generated from the weights."""
+        """Spectra of filter_fn (and filter_fn2) for sequence length L, generated from the weights.
+
+        The reference regenerates its filters in every forward and so does this by default.  With
+        `self.cache_filters = True` (inference with frozen weights) the spectra are kept and reused until a
+        filter parameter or buffer changes (in-place updates bump the tensor version; re-assignment changes
+        the storage pointer)."""
         fns = [self.filter_fn] + ([self.filter_fn2] if self.residual_long_conv else [])
+        if self.cache_filters:
+            tag = (L,) + tuple((t.data_ptr(), t._version) for f in fns
+                               for t in list(f.parameters()) + list(f.buffers()))
+            hit = self._spec_cache
+            if hit is not None and hit[0] == tag:
+                return hit[1]
+            spec = self._generate_spectrum(L, fns)
+            self._spec_cache = (tag, spec)
+            return spec
+        return self._generate_spectrum(L, fns)
+
+    def _generate_spectrum(self, L: int, fns) -> torch.Tensor:
         f0 = self.filter_fn
         taps = ops.hyena_filter_taps([f.kernel_params("both") for f in fns], L, self.d_model, f0.order, f0.emb_dim,
                                      w_mod=float(f0.w_mod), shift=float(f0.modulation.shift))

@@ -214,3 +214,28 @@ def test_encoder_hip_graph_replays_match_eager(gpu):
     assert len(graphed.encoder._graphs) == 2
     graphed.encoder.reset_graphs()
     assert len(graphed.encoder._graphs) == 0
+
+
+def test_cached_filter_spectra_follow_the_weights(gpu):
+    """cache_filters=True reuses the spectra and regenerates them when a filter weight changes."""
+    import m2_amd
+    cfg = m2_amd.m2_bert_80m(128)
+    sd = m2_amd.seeded_state_dict(cfg, 3, what="mixer")
+    mix = m2_amd.MonarchMixerSequenceMixing(768, l_max=128, bidirectional=True, hyena_emb_dim=5, hyena_filter_order=128,
+                                            residual_long_conv=True, hyena_w=10)
+    mix.load_state_dict(sd)
+    mix = mix.to(gpu).eval()
+    u = torch.randn(2, 128, 768, generator=torch.Generator().manual_seed(1)).to(gpu)
+    y0, _ = mix(u)
+    mix.cache_filters = True
+    y1, _ = mix(u)
+    spec_a = mix._spec_cache[1]
+    y2, _ = mix(u)
+    assert mix._spec_cache[1] is spec_a and torch.equal(y0, y1) and torch.equal(y1, y2)
+    with torch.no_grad():
+        mix.filter_fn.bias.add_(1.0)                       # the skip weight D1 is part of the spectrum
+    y3, _ = mix(u)
+    assert mix._spec_cache[1] is not spec_a and not torch.equal(y3, y2)
+    mix.cache_filters = False
+    y4, _ = mix(u)
+    assert torch.equal(y3, y4)
