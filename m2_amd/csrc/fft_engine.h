@@ -29,6 +29,11 @@ struct Plan {
   static constexpr int RL = (R3 > 1) ? R3 : R2;   // radix of the least significant digit of a group index
   static constexpr int WG = T < 256 ? 256 : T;    // threads per workgroup
   static constexpr int RPW = WG / T;              // rows per workgroup
+  // Pass-1 twiddles: kept in registers for the whole kernel when the register budget allows it
+  // (up to 512 threads per workgroup), else only the base roots are kept and the powers are rebuilt
+  // where they are used (a 1024-thread workgroup has 128 registers per thread, and 30 long-lived
+  // twiddle registers would be spilled to memory and re-read for every row).
+  static constexpr bool P1_REGS = WG < 1024;
   static constexpr int ROW_LDS = N + (N >> 4);    // padded complex slots per row
   static constexpr int TW_LDS = R2 * (N / R1 / R2) + (R3_ > 1 ? R3_ * (N / R1 / R2 / R3_) : 0);   // twiddle tables
   static constexpr int WG_LDS = (T < 256 ? 256 / T : 1) * ROW_LDS + TW_LDS;                         // float2 slots per workgroup
@@ -66,7 +71,7 @@ __device__ __forceinline__ cf unit_root(int m, int n) {
 // pass: tables in LDS ([k][m], conflict-free for consecutive m), built once per workgroup.
 template <class P>
 struct Twiddles {
-  cf p1[16 / P::R1][P::R1];     // [butterfly][k], k = 1 .. R1-1
+  cf p1[16 / P::R1][P::P1_REGS ? P::R1 : 2];     // [butterfly][k], k = 1 .. R1-1 (k = 1 only without P1_REGS)
   const float2* tab2;           // [R2][S2]
   const float2* tab3;           // [R3][S3]   (R3 > 1 only)
   static constexpr int TAB2 = P::R2 * P::S2;
@@ -81,7 +86,9 @@ __device__ __forceinline__ void twiddles_init(Twiddles<P>& tw, int t, float2* ta
   static_for<0, NB>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
     const int q = t + P::T * i;
-    powers<P::R1>(unit_root(q % P::S1, P::S1 * P::R1), tw.p1[i]);
+    const cf w = unit_root(q % P::S1, P::S1 * P::R1);
+    if constexpr (P::P1_REGS) powers<P::R1>(w, tw.p1[i]);
+    else tw.p1[i][1] = w;
   });
   tw.tab2 = tables;
   tw.tab3 = tables + Twiddles<P>::TAB2;
@@ -100,15 +107,24 @@ __device__ __forceinline__ void twiddles_init(Twiddles<P>& tw, int t, float2* ta
   __syncthreads();
 }
 
-// twiddle w^(m k) of pass PASS (1, 2 or 3) for butterfly i of this thread
-template <class P, int PASS, int S, int I, int K>
-__device__ __forceinline__ cf pass_twiddle(const Twiddles<P>& tw, int m) {
-  if constexpr (PASS == 1) {
-    return tw.p1[I][K];
+// pass-1 twiddles pw[k] = w^k of butterfly I of this thread
+template <class P, int I>
+__device__ __forceinline__ void pass1_twiddles(const Twiddles<P>& tw, cf (&pw)[P::R1]) {
+  if constexpr (P::P1_REGS) {
+    static_for<1, P::R1>([&](auto k) { pw[decltype(k)::value] = tw.p1[I][decltype(k)::value]; });
   } else {
-    const float2 v = (PASS == 2 ? tw.tab2 : tw.tab3)[K * S + m];
-    return {v.x, v.y};
+    cf w = tw.p1[I][1];
+    // opaque to the optimiser, so that the powers are rebuilt here and not hoisted out of the row loop
+    asm volatile("" : "+v"(w.re), "+v"(w.im));
+    powers<P::R1>(w, pw);
   }
+}
+
+// twiddle w^(m k) of pass PASS (2 or 3), shared table in LDS
+template <class P, int PASS, int S, int K>
+__device__ __forceinline__ cf table_twiddle(const Twiddles<P>& tw, int m) {
+  const float2 v = (PASS == 2 ? tw.tab2 : tw.tab3)[K * S + m];
+  return {v.x, v.y};
 }
 
 // forward: registers hold natural-order inputs of E/R butterflies; butterfly, twiddle, store.
@@ -123,10 +139,15 @@ __device__ __forceinline__ void fwd_compute_store(cf (&x)[16], int t, float2* ro
     else dif<R, i * R, 16>(x);
     float2* pb = row + phys(b * (S * R) + m);
     constexpr int bits = ilog2(R);
+    cf pw[PASS == 1 ? P::R1 : 1];
+    if constexpr (PASS == 1) pass1_twiddles<P, i>(tw, pw);
     static_for<0, R>([&](auto kk) {
       constexpr int k = decltype(kk)::value;
       cf v = x[i * R + bitrev(k, bits)];
-      if constexpr (k > 0) v = cmul(v, pass_twiddle<P, PASS, S, i, k>(tw, m));
+      if constexpr (k > 0) {
+        if constexpr (PASS == 1) v = cmul(v, pw[k]);
+        else v = cmul(v, table_twiddle<P, PASS, S, k>(tw, m));
+      }
       lds_put(pb, poff(k * S), v);
     });
   });
@@ -157,10 +178,15 @@ __device__ __forceinline__ void inv_load_compute(cf (&x)[16], int t, const float
     const int b = q / S, m = q % S;
     const float2* pb = row + phys(b * (S * R) + m);
     constexpr int bits = ilog2(R);
+    cf pw[PASS == 1 ? P::R1 : 1];
+    if constexpr (PASS == 1) pass1_twiddles<P, i>(tw, pw);
     static_for<0, R>([&](auto kk) {
       constexpr int k = decltype(kk)::value;
       cf v = lds_get(pb, poff(k * S));
-      if constexpr (k > 0) v = cmulc(v, pass_twiddle<P, PASS, S, i, k>(tw, m));
+      if constexpr (k > 0) {
+        if constexpr (PASS == 1) v = cmulc(v, pw[k]);
+        else v = cmulc(v, table_twiddle<P, PASS, S, k>(tw, m));
+      }
       x[i * R + bitrev(k, bits)] = v;
     });
     if constexpr (LOWER_ONLY) dit_lower_only<R, i * R, 16>(x);
