@@ -137,31 +137,60 @@ __device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, 
   return __builtin_bit_cast(bf16x8, v);
 }
 
-// Workgroup = 4 waves; wave w owns channels [c0 + 64 w, +64) with its weight rows split into bf16
-// hi / lo parts held in registers, and walks kPosPerWg positions in tiles of 32.
-// grid (L / kPosPerWg, d / 256 rounded up, 2 * nfilters).
+// Workgroup = 4 waves = 128 channels; wave w owns channels [c0 + 32 w, + 32) with its weight rows split
+// into bf16 hi / lo parts held in registers.  The workgroup walks kPosPerWg positions in tiles of 32:
+// the h3 tile (hi and lo parts, 16 KB) is fetched with coalesced 16-byte loads one tile ahead, staged in
+// LDS (double buffered, rows padded to 272 bytes so that the 16-byte operand reads of 32 rows spread over
+// all banks) and shared by the four waves.
+// grid (L / kPosPerWg rounded up, d / 128 rounded up, 2 * nfilters).
 constexpr int kPosPerWg = 256;      // at most; 32-position tiles past L are skipped
-__global__ __launch_bounds__(256) void project_kernel(FilterBatch fb, int L, int d, float shift,
+constexpr int kHRow = 2 * kOrder + 16;   // bytes per padded LDS row of one h3 part
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) void project_kernel(FilterBatch fb, int L, int d, float shift,
                                                       const uint16_t* __restrict__ h_hi, const uint16_t* __restrict__ h_lo,
                                                       float* __restrict__ taps /* (nf, d, 2L) */) {
+  __shared__ __attribute__((aligned(16))) unsigned char hbuf[2][2][32 * kHRow];     // [buffer][hi, lo][row]
   const int fi = blockIdx.z >> 1, dir = blockIdx.z & 1;
   const FilterPtrs& F = fb.f[fi];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
-  const int c0 = blockIdx.y * 256 + wave * 64;
-  if (c0 >= d) return;
+  const int c0 = blockIdx.y * 128 + wave * 32;
+  const bool active = c0 < d;                      // d is a multiple of 64: a wave is all in or all out
   const int lbase = blockIdx.x * kPosPerWg;
   float* out = taps + (long)fi * d * 2 * L;
   if (F.mlp[dir].w3 == nullptr) {
     // not bidirectional: the reverse half of the window is zero
-    for (int r = 0; r < 64; ++r)
-      for (int p = lane; p < kPosPerWg && lbase + p < L; p += 64) out[(long)(c0 + r) * 2 * L + L + lbase + p] = 0.f;
+    if (active)
+      for (int r = 0; r < 32; ++r)
+        for (int p = lane; p < kPosPerWg && lbase + p < L; p += 64) out[(long)(c0 + r) * 2 * L + L + lbase + p] = 0.f;
     return;
   }
-  // A operand: rows c0 + 32 a + i32, K = 16 ks + 8 half + {0..7}, split hi / lo
-  bf16x8 ahi[2][kOrder / 16], alo[2][kOrder / 16];
-#pragma unroll
-  for (int a = 0; a < 2; ++a) {
-    const float* wr = F.mlp[dir].w3 + (long)(c0 + 32 * a + i32) * kOrder + 8 * half;
+  int ntiles = (L - lbase) / 32;
+  if (ntiles > kPosPerWg / 32) ntiles = kPosPerWg / 32;
+
+  // staging: thread -> two 16-byte pieces of each part of the (contiguous, 8 KB) tile
+  const long tile_elems = 32L * kOrder;
+  const uint16_t* gh = h_hi + ((long)blockIdx.z * L + lbase) * kOrder + 8 * tid;
+  const uint16_t* gl = h_lo + ((long)blockIdx.z * L + lbase) * kOrder + 8 * tid;
+  const int srow0 = tid >> 4, scol = (tid & 15) * 16;              // piece q covers row srow0 + 16 q
+  u32x4 st[4];
+  auto fetch = [&](int pt) __attribute__((always_inline)) {
+    st[0] = *reinterpret_cast<const u32x4*>(gh + pt * tile_elems);
+    st[1] = *reinterpret_cast<const u32x4*>(gh + pt * tile_elems + 16 * kOrder);
+    st[2] = *reinterpret_cast<const u32x4*>(gl + pt * tile_elems);
+    st[3] = *reinterpret_cast<const u32x4*>(gl + pt * tile_elems + 16 * kOrder);
+  };
+  auto stage = [&](int buf) __attribute__((always_inline)) {
+    *reinterpret_cast<u32x4*>(&hbuf[buf][0][srow0 * kHRow + scol]) = st[0];
+    *reinterpret_cast<u32x4*>(&hbuf[buf][0][(srow0 + 16) * kHRow + scol]) = st[1];
+    *reinterpret_cast<u32x4*>(&hbuf[buf][1][srow0 * kHRow + scol]) = st[2];
+    *reinterpret_cast<u32x4*>(&hbuf[buf][1][(srow0 + 16) * kHRow + scol]) = st[3];
+  };
+  fetch(0);
+
+  // A operand: rows c0 + i32, K = 16 ks + 8 half + {0..7}, split hi / lo
+  bf16x8 ahi[kOrder / 16], alo[kOrder / 16];
+  float adelta[16];
+  if (active) {
+    const float* wr = F.mlp[dir].w3 + (long)(c0 + i32) * kOrder + 8 * half;
 #pragma unroll
     for (int ks = 0; ks < kOrder / 16; ++ks) {
       const float4 v0 = *reinterpret_cast<const float4*>(wr + 16 * ks);
@@ -173,47 +202,45 @@ __global__ __launch_bounds__(256) void project_kernel(FilterBatch fb, int L, int
         h[j] = bf16_to_f32(f32_to_bf16(x[j]));
         l[j] = x[j] - h[j];
       }
-      ahi[a][ks] = as_bf16x8(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]), pack_bf16x2(h[4], h[5]), pack_bf16x2(h[6], h[7]));
-      alo[a][ks] = as_bf16x8(pack_bf16x2(l[0], l[1]), pack_bf16x2(l[2], l[3]), pack_bf16x2(l[4], l[5]), pack_bf16x2(l[6], l[7]));
+      ahi[ks] = as_bf16x8(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]), pack_bf16x2(h[4], h[5]), pack_bf16x2(h[6], h[7]));
+      alo[ks] = as_bf16x8(pack_bf16x2(l[0], l[1]), pack_bf16x2(l[2], l[3]), pack_bf16x2(l[4], l[5]), pack_bf16x2(l[6], l[7]));
     }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) adelta[v] = -fabsf(F.deltas[c0 + 8 * (v >> 2) + 4 * half + (v & 3)]) * 1.44269504088896341f;
   }
-  float adelta[2][16];
-#pragma unroll
-  for (int a = 0; a < 2; ++a)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) adelta[a][v] = -fabsf(F.deltas[c0 + 32 * a + 8 * (v >> 2) + 4 * half + (v & 3)]) * 1.44269504088896341f;
+  stage(0);
+  __syncthreads();
 
-  const uint16_t* bh = h_hi + ((long)blockIdx.z * L + lbase + i32) * kOrder + 8 * half;
-  const uint16_t* bl = h_lo + ((long)blockIdx.z * L + lbase + i32) * kOrder + 8 * half;
-  for (int pt = 0; pt < kPosPerWg / 32 && lbase + pt * 32 < L; ++pt) {
-    floatx16 acc[2];
+  for (int pt = 0; pt < ntiles; ++pt) {
+    if (pt + 1 < ntiles) fetch(pt + 1);
+    if (active) {
+      const unsigned char* bh = &hbuf[pt & 1][0][i32 * kHRow + 16 * half];
+      const unsigned char* bl = &hbuf[pt & 1][1][i32 * kHRow + 16 * half];
+      floatx16 acc;
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+      for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[a][v] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < kOrder / 16; ++ks) {
-      const bf16x8 bhi = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(bh + (long)pt * 32 * kOrder + 16 * ks));
-      const bf16x8 blo = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(bl + (long)pt * 32 * kOrder + 16 * ks));
-#pragma unroll
-      for (int a = 0; a < 2; ++a) {
-        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[a][ks], bhi, acc[a], 0, 0, 0);
-        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[a][ks], blo, acc[a], 0, 0, 0);
-        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[a][ks], bhi, acc[a], 0, 0, 0);
+      for (int ks = 0; ks < kOrder / 16; ++ks) {
+        const bf16x8 bhi = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(bh + 32 * ks));
+        const bf16x8 blo = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(bl + 32 * ks));
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[ks], bhi, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[ks], blo, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[ks], bhi, acc, 0, 0, 0);
       }
-    }
-    // accumulator element v of lane: channel c0 + 32 a + 8 (v / 4) + 4 half + v % 4, position i32
-    const int l = lbase + pt * 32 + i32;
-    const float tl = F.t[l];
-    const long pos = dir == 0 ? l : (2L * L - 1 - l);
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
+      // accumulator element v of lane: channel c0 + 8 (v / 4) + 4 half + v % 4, position i32
+      const int l = lbase + pt * 32 + i32;
+      const float tl = F.t[l];
+      float* po = out + (long)(c0 + 4 * half) * 2 * L + (dir == 0 ? l : (2L * L - 1 - l));
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int c = c0 + 32 * a + 8 * (v >> 2) + 4 * half + (v & 3);
-        const float decay = exp2f(tl * adelta[a][v]) + shift;        // exp(-t |delta|)
-        out[(long)c * 2 * L + pos] = acc[a][v] * decay;
+        // exp(-t |delta|); the bare hardware exp2 flushes results below 2^-126 to zero, which is the
+        // value to 1e-38 absolute
+        const float decay = __builtin_amdgcn_exp2f(tl * adelta[v]) + shift;
+        po[(long)(8 * (v >> 2) + (v & 3)) * 2 * L] = acc[v] * decay;
       }
+    }
+    if (pt + 1 < ntiles) stage((pt + 1) & 1);
+    __syncthreads();
   }
 }
 
@@ -257,7 +284,7 @@ extern "C" int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfi
   hipLaunchKernelGGL(hidden_kernel, dim3(L / kPosTile, 2 * nfilters), dim3(256), 0, s, fb, L, emb_dim, w_mod, h_hi, h_lo);
   int rc = check_launch("hyena hidden_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL(project_kernel, dim3((L + kPosPerWg - 1) / kPosPerWg, (d + 255) / 256, 2 * nfilters), dim3(256), 0, s, fb, L, d, shift,
+  hipLaunchKernelGGL(project_kernel, dim3((L + kPosPerWg - 1) / kPosPerWg, (d + 127) / 128, 2 * nfilters), dim3(256), 0, s, fb, L, d, shift,
                      h_hi, h_lo, taps);
   return check_launch("hyena project_kernel");
 }
