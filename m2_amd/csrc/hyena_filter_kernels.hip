@@ -72,16 +72,25 @@ __global__ __launch_bounds__(256) void hidden_kernel(FilterBatch fb, int L, int 
   if (W.w0 == nullptr) return;                  // not bidirectional: nothing to do for dir == 1
   const int l0 = blockIdx.x * kPosTile;
 
-  // layer 0 (emb -> 128) on the vector ALU: thread = (neuron o, 16 positions)
+  // layer 0 (emb -> 128) on the vector ALU: thread = (neuron o, 16 positions).  The tile's embeddings
+  // (32 x emb consecutive floats) go through LDS; weights beyond emb are zero so the dot product has a
+  // fixed length.
   {
+    __shared__ float zt[kPosTile * kMaxEmb];
+    zt[tid] = tid < kPosTile * emb ? F.z[(long)l0 * emb + tid] : 0.f;
     const int o = tid & (kOrder - 1), p0 = (tid >> 7) * 16;
     float w[kMaxEmb];
+#pragma unroll
     for (int e = 0; e < kMaxEmb; ++e) w[e] = e < emb ? W.w0[o * emb + e] : 0.f;
     const float b = W.b0[o], fo = w_mod * F.freq[o];
-    for (int p = p0; p < p0 + 16; ++p) {
-      const float* zp = F.z + (long)(l0 + p) * emb;
+    __syncthreads();
+#pragma unroll
+    for (int pp = 0; pp < 16; ++pp) {
+      const int p = p0 + pp;
+      const int zi = p * emb;
       float acc = b;
-      for (int e = 0; e < emb; ++e) acc += w[e] * zp[e];
+#pragma unroll
+      for (int e = 0; e < kMaxEmb; ++e) acc += w[e] * zt[zi + e];      // zi + e <= 31 emb + 7 < 256
       act[0][p][o] = sin_reduced(fo * acc);
     }
   }
@@ -112,9 +121,12 @@ __global__ __launch_bounds__(256) void hidden_kernel(FilterBatch fb, int L, int 
 #pragma unroll
     for (int vq = 0; vq < 4; ++vq) {
       const int o = 32 * wave + 8 * vq + 4 * half;
+      const float4 fq = *reinterpret_cast<const float4*>(F.freq + o);
+      const float4 bq = *reinterpret_cast<const float4*>(bias + o);
+      const float fr[4] = {fq.x, fq.y, fq.z, fq.w}, bs[4] = {bq.x, bq.y, bq.z, bq.w};
       float s[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s[j] = sin_reduced(w_mod * F.freq[o + j] * (acc[4 * vq + j] + bias[o + j]));
+      for (int j = 0; j < 4; ++j) s[j] = sin_reduced(w_mod * fr[j] * (acc[4 * vq + j] + bs[j]));
       if (layer == 0) {
         *reinterpret_cast<float4*>(&act[dst][i32][o]) = make_float4(s[0], s[1], s[2], s[3]);
       } else {
