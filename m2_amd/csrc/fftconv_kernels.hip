@@ -34,52 +34,13 @@
 #include <stdint.h>
 
 #include "fft_engine.h"
+#include "row_io.h"
 
 namespace m2 {
 
 // ------------------------------------------------------------------------------------------
 // K2: the fused mixer core
 // ------------------------------------------------------------------------------------------
-// 8 consecutive activations starting at element n0 (n0 % 8 == 0) plus the two before them, as fp32:
-// out[0], out[1] = in[n0-2], in[n0-1] (zero when n0 == 0), out[2..10) = in[n0 .. n0+8).
-// `add` is added to every element that exists (the two before n0 == 0 stay zero: that is the
-// convolution's zero padding, which sits outside the biased signal).
-__device__ __forceinline__ void load10(const float* p, int n0, float add, float (&o)[10]) {
-  const float4 a = *reinterpret_cast<const float4*>(p + n0);
-  const float4 b = *reinterpret_cast<const float4*>(p + n0 + 4);
-  o[0] = 0.f; o[1] = 0.f;
-  if (n0 > 0) {
-    const float2 h = *reinterpret_cast<const float2*>(p + n0 - 2);
-    o[0] = h.x + add; o[1] = h.y + add;
-  }
-  o[2] = a.x + add; o[3] = a.y + add; o[4] = a.z + add; o[5] = a.w + add;
-  o[6] = b.x + add; o[7] = b.y + add; o[8] = b.z + add; o[9] = b.w + add;
-}
-__device__ __forceinline__ void load10(const uint16_t* p, int n0, float add, float (&o)[10]) {
-  const uint4 a = *reinterpret_cast<const uint4*>(p + n0);
-  o[0] = 0.f; o[1] = 0.f;
-  if (n0 > 0) {
-    const uint32_t h = *reinterpret_cast<const uint32_t*>(p + n0 - 2);
-    o[0] = __uint_as_float(h << 16) + add; o[1] = __uint_as_float(h & 0xffff0000u) + add;
-  }
-  o[2] = __uint_as_float(a.x << 16) + add; o[3] = __uint_as_float(a.x & 0xffff0000u) + add;
-  o[4] = __uint_as_float(a.y << 16) + add; o[5] = __uint_as_float(a.y & 0xffff0000u) + add;
-  o[6] = __uint_as_float(a.z << 16) + add; o[7] = __uint_as_float(a.z & 0xffff0000u) + add;
-  o[8] = __uint_as_float(a.w << 16) + add; o[9] = __uint_as_float(a.w & 0xffff0000u) + add;
-}
-__device__ __forceinline__ void store8(float* p, int n0, const float (&v)[8]) {
-  *reinterpret_cast<float4*>(p + n0) = make_float4(v[0], v[1], v[2], v[3]);
-  *reinterpret_cast<float4*>(p + n0 + 4) = make_float4(v[4], v[5], v[6], v[7]);
-}
-__device__ __forceinline__ void store8(uint16_t* p, int n0, const float (&v)[8]) {
-  uint4 o;
-  o.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
-  o.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
-  o.z = (uint32_t)f32_to_bf16(v[4]) | ((uint32_t)f32_to_bf16(v[5]) << 16);
-  o.w = (uint32_t)f32_to_bf16(v[6]) | ((uint32_t)f32_to_bf16(v[7]) << 16);
-  *reinterpret_cast<uint4*>(p + n0) = o;
-}
-
 // first forward pass when only positions [0, N/2) of the row are populated (upper half is zero)
 template <class P>
 __device__ __forceinline__ void fwd_load_lower(cf (&x)[16], int t, const float2* row) {
@@ -377,6 +338,13 @@ int launch_mixer_core_big_dispatch(const void* xproj, const float* u, const floa
 int launch_filter_spectrum_big(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
                                int d, hipStream_t stream);
 
+// L = 4096, 8192: even/odd split half transforms, defined in fftconv_split_kernels.hip
+bool split_plan_exists(int L);
+int launch_mixer_split_dispatch(const void* xproj, const float* u, const float* sw, const float* sb, const float* pbias,
+                                const float* spec, void* y, int B, int L, int d, int act_dtype, hipStream_t stream);
+int launch_filter_spectrum_split(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
+                                 int d, int L, hipStream_t stream);
+
 }  // namespace m2
 
 using namespace m2;
@@ -398,6 +366,7 @@ extern "C" int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, co
     return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: L=%d unsupported (need 2L a power of two in [256, 16384], or 65536)", L);
   const int logn = ilog2(2 * L);
   if (logn == 16) return launch_filter_spectrum_big(taps1, taps2, D1, D2, spec, d, (hipStream_t)stream);
+  if (split_plan_exists(L)) return launch_filter_spectrum_split(taps1, taps2, D1, D2, spec, d, L, (hipStream_t)stream);
   switch (logn) {
 #define X(LOGN, R1, R2, R3) \
   case LOGN:                \
@@ -420,6 +389,7 @@ extern "C" int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, cons
   const int logn = ilog2(2 * L);
   hipStream_t s = (hipStream_t)stream;
   if (logn == 16) return launch_mixer_core_big_dispatch(xproj, u, short_w, short_b, proj_bias, spec, y, B, d, act_dtype, s);
+  if (split_plan_exists(L)) return launch_mixer_split_dispatch(xproj, u, short_w, short_b, proj_bias, spec, y, B, L, d, act_dtype, s);
   switch (logn) {
 #define X(LOGN, R1, R2, R3)                                                                                       \
   case LOGN:                                                                                                      \
@@ -443,6 +413,7 @@ extern "C" int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, 
   const int logn = ilog2(2 * L);
   hipStream_t s = (hipStream_t)stream;
   if (logn == 16) return launch_mixer_core_big_dispatch(x, nullptr, nullptr, nullptr, nullptr, spec, y, B, d, act_dtype, s);
+  if (split_plan_exists(L)) return launch_mixer_split_dispatch(x, nullptr, nullptr, nullptr, nullptr, spec, y, B, L, d, act_dtype, s);
   switch (logn) {
 #define X(LOGN, R1, R2, R3)                                                                                  \
   case LOGN:                                                                                                 \
