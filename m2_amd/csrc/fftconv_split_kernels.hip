@@ -296,6 +296,17 @@ __device__ __forceinline__ void split_groups(int w, int& g, int& g_mirror, int& 
   g_mirror = k1 * R2 + k2;
 }
 
+// One spectral pair: za sits at frequency kappa, zb at N - kappa.  Returns W[kappa] in za and W[N - kappa] in
+// zb.  The 1/2 of the even/odd separation is folded into the stored spectra.
+__device__ __forceinline__ void pair_multiply_half(cf& za, cf& zb, float4 K) {
+  const cf A = {za.re + zb.re, za.im - zb.im};         // Z[k] + conj Z[N-k]
+  const cf Bq = {za.im + zb.im, zb.re - za.re};        // (Z[k] - conj Z[N-k]) / i
+  const cf Pp = cmul(A, cf{K.x, K.y});
+  const cf Q = cmul(Bq, cf{K.z, K.w});
+  za = {Pp.re - Q.im, Pp.im + Q.re};                   // P + iQ
+  zb = {Pp.re + Q.im, Q.re - Pp.im};                   // conj(P) + i conj(Q)
+}
+
 // spectral multiply of the 16 + 16 points a thread holds after fwd_groups, slots 8 H .. 8 H + 7.
 // EVEN_SPECIAL: this is work item 0 of the even half (DC, Nyquist and the two self-mirrored groups).
 template <bool EVEN_SPECIAL, int H>
@@ -304,15 +315,15 @@ __device__ __forceinline__ void multiply_batch(cf (&x)[32], const float4 (&K)[8]
     constexpr int s = 8 * H + decltype(ss)::value;
     const float4 k = K[decltype(ss)::value];
     if constexpr (!EVEN_SPECIAL) {
-      pair_multiply(x[bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], k);
+      pair_multiply_half(x[bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], k);
     } else if constexpr (s == 0) {
       // DC and Nyquist are self-paired and their filter values are real: K = (K1(0), K1(N/2), K2(0), K2(N/2))
       x[bitrev(0, 4)] = {x[bitrev(0, 4)].re * k.x, x[bitrev(0, 4)].im * k.z};
       x[bitrev(8, 4)] = {x[bitrev(8, 4)].re * k.y, x[bitrev(8, 4)].im * k.w};
     } else if constexpr (s < 8) {
-      pair_multiply(x[bitrev(s, 4)], x[bitrev(16 - s, 4)], k);              // group 0: slot s <-> 16 - s
+      pair_multiply_half(x[bitrev(s, 4)], x[bitrev(16 - s, 4)], k);              // group 0: slot s <-> 16 - s
     } else {
-      pair_multiply(x[16 + bitrev(s - 8, 4)], x[16 + bitrev(23 - s, 4)], k);   // group R2/2: slot j <-> 15 - j
+      pair_multiply_half(x[16 + bitrev(s - 8, 4)], x[16 + bitrev(23 - s, 4)], k);   // group R2/2: slot j <-> 15 - j
     }
   });
 }
@@ -544,7 +555,9 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_split_kernel(
   static_for<0, P::NB1>([&](auto ii) { b[decltype(ii)::value] = unit_root(t + T * decltype(ii)::value, P::N); });
   int g, gm, gc;
   split_groups<P>(t, g, gm, gc);
-  const float scale = 0.5f / (float)N;       // the 1/2 of the even/odd split and the 1/N of the convolution
+  // 1/N of the convolution, 1/2 of the separation of the two packed filters, 1/2 of the separation of the two
+  // packed signals in the mixer kernel (pair_multiply_half)
+  const float scale = 0.25f / (float)N;
   __syncthreads();
 
   auto split = [&](cf za, cf zb) __attribute__((always_inline)) -> float4 {
@@ -601,7 +614,7 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_split_kernel(
       float4* sp = spec + ((long)c * 2 + (ODD ? 1 : 0)) * 16 * T + t;
       if (!ODD && t == 0) {
         const cf z0 = x[bitrev(0, 4)], zn = x[bitrev(8, 4)];
-        sp[0] = make_float4(2.f * scale * z0.re, 2.f * scale * zn.re, 2.f * scale * z0.im, 2.f * scale * zn.im);
+        sp[0] = make_float4(4.f * scale * z0.re, 4.f * scale * zn.re, 4.f * scale * z0.im, 4.f * scale * zn.im);
         static_for<1, 8>([&](auto ss) {
           constexpr int s = decltype(ss)::value;
           sp[s * T] = split(x[bitrev(s, 4)], x[bitrev(16 - s, 4)]);

@@ -70,11 +70,23 @@ class BertEmbeddings(nn.Module):
                 past_key_values_length: int = 0) -> torch.Tensor:
         if self.training and self.dropout.p > 0:
             raise NotImplementedError("m2_amd is a forward/inference path: call .eval() first")
+        o32, _, _ = self.forward_forms(input_ids, token_type_ids, position_ids, inputs_embeds, past_key_values_length,
+                                       want_f32=True, want_bf16=False, want_channel_major=False)
+        return o32
+
+    def forward_forms(self, input_ids=None, token_type_ids=None, position_ids=None, inputs_embeds=None,
+                      past_key_values_length: int = 0, want_f32: bool = True, want_bf16: bool = True,
+                      want_channel_major: bool = True):
+        """The embedding LayerNorm written in the forms the first encoder layer reads, by one kernel:
+        (B, L, d) fp32 | (B*L, d) bf16 | (d, B*L) fp32; forms not asked for are None."""
+        if self.training and self.dropout.p > 0:
+            raise NotImplementedError("m2_amd is a forward/inference path: call .eval() first")
         e = self.summed(input_ids, token_type_ids, position_ids, inputs_embeds, past_key_values_length).float()
         B, L, d = e.shape
-        o32, _, _ = ops.layernorm(e.reshape(B * L, d).contiguous(), self.LayerNorm.weight.detach().float(),
-                                  self.LayerNorm.bias.detach().float(), self.LayerNorm.eps)
-        return o32.view(B, L, d)
+        o32, o16, oT = ops.layernorm(e.reshape(B * L, d).contiguous(), self.LayerNorm.weight.detach().float(),
+                                     self.LayerNorm.bias.detach().float(), self.LayerNorm.eps, want_f32=want_f32,
+                                     want_bf16=want_bf16, want_channel_major=want_channel_major)
+        return (None if o32 is None else o32.view(B, L, d)), o16, oT
 
 
 class BertGatedLinearUnitMLP(nn.Module):
@@ -174,11 +186,16 @@ class BertEncoder(nn.Module):
         return super().load_state_dict(*args, **kwargs)
 
     # -- the fused schedule --------------------------------------------------------------------
-    def _run_layers(self, h32: torch.Tensor, B: int, L: int, all_layers: bool) -> List[torch.Tensor]:
-        """h32 (M, d) fp32 contiguous -> list of (M, d) fp32: every layer's output, or only the last."""
+    def _run_layers(self, h32: Optional[torch.Tensor], B: int, L: int, all_layers: bool,
+                    h16: Optional[torch.Tensor] = None, hT: Optional[torch.Tensor] = None) -> List[torch.Tensor]:
+        """h32 (M, d) fp32 contiguous -> list of (M, d) fp32: every layer's output, or only the last.  A caller
+        that already holds the bf16 and the channel-major fp32 form of the input passes them as h16 / hT (and
+        may then pass h32 = None)."""
         with torch.autocast("cuda", enabled=False):
-            h16 = h32.to(torch.bfloat16)
-            hT = h32.t().contiguous()
+            if h16 is None:
+                h16 = h32.to(torch.bfloat16)
+            if hT is None:
+                hT = h32.t().contiguous()
             outs = []
             n = len(self.layer)
             o32 = h32
@@ -189,24 +206,28 @@ class BertEncoder(nn.Module):
                     outs.append(o32)
         return outs
 
-    def _run_graphed(self, h32: torch.Tensor, B: int, L: int, all_layers: bool) -> List[torch.Tensor]:
-        key = (B, L, h32.shape[1], all_layers, h32.device)
+    def _run_graphed(self, h32: Optional[torch.Tensor], B: int, L: int, all_layers: bool,
+                     h16: Optional[torch.Tensor] = None, hT: Optional[torch.Tensor] = None) -> List[torch.Tensor]:
+        given = [t for t in (h32, h16, hT) if t is not None]
+        key = (B, L, given[0].shape[-1] if h32 is not None else h16.shape[-1], all_layers, given[0].device,
+               h32 is None, h16 is None, hT is None)
         entry = self._graphs.get(key)
         if entry is None:
-            static_in = torch.empty_like(h32)
-            static_in.copy_(h32)
+            static = [None if t is None else t.clone() for t in (h32, h16, hT)]
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):                  # warm-up outside the capture (allocator, lazy inits)
-                self._run_layers(static_in, B, L, all_layers)
+                self._run_layers(static[0], B, L, all_layers, h16=static[1], hT=static[2])
             torch.cuda.current_stream().wait_stream(side)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                static_out = self._run_layers(static_in, B, L, all_layers)
-            entry = (graph, static_in, static_out)
+                static_out = self._run_layers(static[0], B, L, all_layers, h16=static[1], hT=static[2])
+            entry = (graph, static, static_out)
             self._graphs[key] = entry
-        graph, static_in, static_out = entry
-        static_in.copy_(h32)
+        graph, static, static_out = entry
+        for dst, src in zip(static, (h32, h16, hT)):
+            if dst is not None:
+                dst.copy_(src)
         graph.replay()
         return [o.clone() for o in static_out]
 
@@ -250,6 +271,9 @@ class BertModel(nn.Module):
                 **kwargs):
         if masked_tokens_mask is not None:
             raise NotImplementedError("masked_tokens_mask subsetting belongs to the MLM head, which is not built")
-        emb = self.embeddings(input_ids, token_type_ids, position_ids)
-        enc = self.encoder(emb, attention_mask, output_all_encoded_layers=output_all_encoded_layers)
+        # the embedding LayerNorm writes the bf16 and channel-major forms the first layer reads itself
+        B, L = input_ids.shape
+        _, h16, hT = self.embeddings.forward_forms(input_ids, token_type_ids, position_ids, want_f32=False)
+        run = self.encoder._run_graphed if self.encoder.use_hip_graph else self.encoder._run_layers
+        enc = [o.view(B, L, -1) for o in run(None, B, L, bool(output_all_encoded_layers), h16=h16, hT=hT)]
         return (enc if output_all_encoded_layers else enc[-1]), None
