@@ -247,90 +247,106 @@ static int launch_blockdiag(const void* x, const void* w, const float* bias, con
 }
 
 // LayerNorm over the last dimension of x (M, d) fp32, eps inside the square root.
-// Workgroup = 16 waves handles 64 rows.  Phase 1: each wave normalises 4 rows at once (all loads in
-// flight together), writes the row-major outputs and leaves mean / rstd in LDS.  Phase 2 re-reads the
-// (cache-resident) rows with lanes along the token axis and writes the channel-major copy with
-// 256-byte stores.  PER = d / 64 values per lane.
+// Workgroup = 8 waves handles R = 8 RW rows; each wave normalises RW rows at once (all loads in flight
+// together) and writes the row-major outputs from registers.  For the channel-major output the
+// normalised rows also go through an LDS tile, 384 columns at a time (row pitch 386 floats, so that 32
+// consecutive tokens of two neighbouring channels fall in 64 different banks; 49 KB, so that three
+// workgroups share a compute unit and one's loads overlap another's stores), and are written back with
+// lanes along the token axis: every store instruction covers R consecutive tokens of 64 / R channels.
+// The input is read once.  PER = d / 64 values per lane.
 template <int PER>
-__global__ __launch_bounds__(1024) void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
-                                                         const float* __restrict__ beta, float eps,
-                                                         float* __restrict__ out_f32,       // (M, d) or null
-                                                         uint16_t* __restrict__ out_bf16,   // (M, d) or null
-                                                         float* __restrict__ out_t,         // (d, M) or null
-                                                         int M) {
-  constexpr int d = 64 * PER;
-  __shared__ float s_mean[64], s_rstd[64];
+struct LnShape {
+  static constexpr int RW = PER <= 16 ? 4 : 2;      // rows in flight per wave (register budget)
+  static constexpr int R = 8 * RW;                  // rows per workgroup: 32 or 16
+  static constexpr int PC = PER < 6 ? PER : 6;      // 64-column groups per tile pass
+  static constexpr int NPASS = (PER + PC - 1) / PC;
+  static constexpr int PITCH = 64 * PC + 2;
+  static constexpr size_t LDS_BYTES = (size_t)R * PITCH * sizeof(float);
+};
+template <int PER>
+__global__ __launch_bounds__(512) void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                                        const float* __restrict__ beta, float eps,
+                                                        float* __restrict__ out_f32,       // (M, d) or null
+                                                        uint16_t* __restrict__ out_bf16,   // (M, d) or null
+                                                        float* __restrict__ out_t,         // (d, M) or null
+                                                        int M) {
+  constexpr int d = 64 * PER, RW = LnShape<PER>::RW, R = LnShape<PER>::R, PITCH = LnShape<PER>::PITCH;
+  constexpr int PC = LnShape<PER>::PC, NPASS = LnShape<PER>::NPASS;
+  extern __shared__ float tile[];                       // [R][PITCH], used only with out_t
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int m0 = blockIdx.x * 64;
-  constexpr int RW = PER <= 16 ? 4 : 2;                 // rows in flight per wave (register budget of 128)
+  const int m0 = blockIdx.x * R;
   float g[PER], bt[PER];
   static_for<0, PER>([&](auto ii) {
     g[decltype(ii)::value] = gamma[lane + 64 * decltype(ii)::value];
     bt[decltype(ii)::value] = beta[lane + 64 * decltype(ii)::value];
   });
-  for (int rb = 0; rb < 4; rb += RW) {
-    float v[RW][PER];
-    float sum[RW], sq[RW];
-    static_for<0, RW>([&](auto rr_) {
-      constexpr int rr = decltype(rr_)::value;
-      int m = m0 + wave * 4 + rb + rr;
-      m = m < M ? m : M - 1;
-      const float* xr = x + (long)m * d;
-      static_for<0, PER>([&](auto ii) { v[rr][decltype(ii)::value] = xr[lane + 64 * decltype(ii)::value]; });
+  float v[RW][PER];
+  float sum[RW], sq[RW];
+  static_for<0, RW>([&](auto rr_) {
+    constexpr int rr = decltype(rr_)::value;
+    int m = m0 + wave * RW + rr;
+    m = m < M ? m : M - 1;
+    const float* xr = x + (long)m * d;
+    static_for<0, PER>([&](auto ii) { v[rr][decltype(ii)::value] = xr[lane + 64 * decltype(ii)::value]; });
+  });
+  static_for<0, RW>([&](auto rr_) {
+    constexpr int rr = decltype(rr_)::value;
+    float s = 0.f;
+    static_for<0, PER>([&](auto ii) { s += v[rr][decltype(ii)::value]; });
+    sum[rr] = s;
+  });
+  for (int o = 32; o > 0; o >>= 1)
+    static_for<0, RW>([&](auto rr_) { sum[decltype(rr_)::value] += __shfl_xor(sum[decltype(rr_)::value], o); });
+  static_for<0, RW>([&](auto rr_) {
+    constexpr int rr = decltype(rr_)::value;
+    sum[rr] *= (1.0f / (float)d);
+    float s = 0.f;
+    static_for<0, PER>([&](auto ii) {
+      const float c = v[rr][decltype(ii)::value] - sum[rr];
+      s += c * c;
     });
-    static_for<0, RW>([&](auto rr_) {
-      constexpr int rr = decltype(rr_)::value;
-      float s = 0.f;
-      static_for<0, PER>([&](auto ii) { s += v[rr][decltype(ii)::value]; });
-      sum[rr] = s;
-    });
-    for (int o = 32; o > 0; o >>= 1)
-      static_for<0, RW>([&](auto rr_) { sum[decltype(rr_)::value] += __shfl_xor(sum[decltype(rr_)::value], o); });
-    static_for<0, RW>([&](auto rr_) {
-      constexpr int rr = decltype(rr_)::value;
-      sum[rr] *= (1.0f / (float)d);
-      float s = 0.f;
-      static_for<0, PER>([&](auto ii) {
-        const float c = v[rr][decltype(ii)::value] - sum[rr];
-        s += c * c;
-      });
-      sq[rr] = s;
-    });
-    for (int o = 32; o > 0; o >>= 1)
-      static_for<0, RW>([&](auto rr_) { sq[decltype(rr_)::value] += __shfl_xor(sq[decltype(rr_)::value], o); });
-    static_for<0, RW>([&](auto rr_) {
-      constexpr int rr = decltype(rr_)::value;
-      const int m = m0 + wave * 4 + rb + rr;
-      const float mean = sum[rr];
-      const float rstd = rsqrtf(sq[rr] * (1.0f / (float)d) + eps);
-      if (lane == 0) { s_mean[wave * 4 + rb + rr] = mean; s_rstd[wave * 4 + rb + rr] = rstd; }
+    sq[rr] = s;
+  });
+  for (int o = 32; o > 0; o >>= 1)
+    static_for<0, RW>([&](auto rr_) { sq[decltype(rr_)::value] += __shfl_xor(sq[decltype(rr_)::value], o); });
+  static_for<0, RW>([&](auto rr_) {
+    constexpr int rr = decltype(rr_)::value;
+    const int m = m0 + wave * RW + rr;
+    const float mean = sum[rr];
+    const float rstd = rsqrtf(sq[rr] * (1.0f / (float)d) + eps);
+    static_for<0, PER>([&](auto ii) {
+      constexpr int i = decltype(ii)::value;
+      v[rr][i] = (v[rr][i] - mean) * rstd * g[i] + bt[i];
       if (m < M) {
-        static_for<0, PER>([&](auto ii) {
-          constexpr int i = decltype(ii)::value;
-          const float o = (v[rr][i] - mean) * rstd * g[i] + bt[i];
-          if (out_f32) out_f32[(long)m * d + lane + 64 * i] = o;
-          if (out_bf16) out_bf16[(long)m * d + lane + 64 * i] = f32_to_bf16(o);
-        });
+        if (out_f32) out_f32[(long)m * d + lane + 64 * i] = v[rr][i];
+        if (out_bf16) out_bf16[(long)m * d + lane + 64 * i] = f32_to_bf16(v[rr][i]);
       }
     });
-  }
+  });
   if (!out_t) return;
-  __syncthreads();
-  const int m = m0 + lane;
-  const bool ok = m < M;
-  const float mean = s_mean[lane], rstd = s_rstd[lane];
-  const float* xr = x + (long)(ok ? m : M - 1) * d;
-  for (int c0 = wave * 4; c0 < d; c0 += 64) {        // 4 channels per wave per step
-    const float4 q = *reinterpret_cast<const float4*>(xr + c0);
-    const float4 g4 = *reinterpret_cast<const float4*>(gamma + c0);
-    const float4 b4 = *reinterpret_cast<const float4*>(beta + c0);
-    if (ok) {
-      out_t[(long)(c0 + 0) * M + m] = (q.x - mean) * rstd * g4.x + b4.x;
-      out_t[(long)(c0 + 1) * M + m] = (q.y - mean) * rstd * g4.y + b4.y;
-      out_t[(long)(c0 + 2) * M + m] = (q.z - mean) * rstd * g4.z + b4.z;
-      out_t[(long)(c0 + 3) * M + m] = (q.w - mean) * rstd * g4.w + b4.w;
+  // lane = (token tk, channel offset h): R tokens x (64 / R) channels per store instruction
+  constexpr int CH = 64 / R;
+  const int tk = lane % R, h = lane / R;
+  const int mt = m0 + tk;
+  static_for<0, NPASS>([&](auto pp) {
+    constexpr int ps = decltype(pp)::value;
+    constexpr int i0 = ps * PC, i1 = (i0 + PC < PER) ? i0 + PC : PER;      // 64-column groups of this pass
+    if (ps > 0) __syncthreads();                                            // the previous pass has been read
+    static_for<0, RW>([&](auto rr_) {
+      constexpr int rr = decltype(rr_)::value;
+      static_for<i0, i1>([&](auto ii) {
+        constexpr int i = decltype(ii)::value;
+        tile[(wave * RW + rr) * PITCH + lane + 64 * (i - i0)] = v[rr][i];
+      });
+    });
+    __syncthreads();
+    if (mt < M) {
+      const float* src = tile + tk * PITCH + h;
+      float* dst = out_t + (long)(64 * i0 + h) * M + mt;
+#pragma unroll 4
+      for (int c0 = wave * CH; c0 < 64 * (i1 - i0); c0 += 8 * CH) dst[(long)c0 * M] = src[c0];
     }
-  }
+  });
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -527,14 +543,21 @@ extern "C" int m2_layernorm_fwd(const float* x, const float* gamma, const float*
   if (!x || !gamma || !beta) return set_error(M2_ERR_ARG, "m2_layernorm_fwd: null pointer");
   if (M <= 0 || d <= 0 || d % 64 != 0 || d > 2048)
     return set_error(M2_ERR_UNSUPPORTED, "m2_layernorm_fwd: need M > 0 and d a multiple of 64 up to 2048 (M=%d d=%d)", M, d);
-  dim3 grid((M + 63) / 64);
   hipStream_t st = (hipStream_t)stream;
   uint16_t* o16 = (uint16_t*)out_bf16;
   switch (d / 64) {
-#define LN_CASE(P)                                                                                                    \
-  case P:                                                                                                             \
-    hipLaunchKernelGGL(layernorm_kernel<P>, grid, dim3(1024), 0, st, x, gamma, beta, eps, out_f32, o16, out_channel_major, M); \
-    break;
+#define LN_CASE(P)                                                                                                      \
+  case P: {                                                                                                             \
+    const size_t lds = out_channel_major ? LnShape<P>::LDS_BYTES : 0;                                                   \
+    auto kern = layernorm_kernel<P>;                                                                                    \
+    if (lds > 64 * 1024) {                                                                                              \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
+      if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(layernorm): %s", hipGetErrorString(e)); \
+    }                                                                                                                   \
+    hipLaunchKernelGGL(kern, dim3((M + LnShape<P>::R - 1) / LnShape<P>::R), dim3(512), lds, st, x, gamma, beta, eps,   \
+                       out_f32, o16, out_channel_major, M);                                                             \
+    break;                                                                                                              \
+  }
     LN_CASE(1) LN_CASE(2) LN_CASE(3) LN_CASE(4) LN_CASE(5) LN_CASE(6) LN_CASE(7) LN_CASE(8) LN_CASE(9) LN_CASE(10) LN_CASE(11)
     LN_CASE(12) LN_CASE(13) LN_CASE(14) LN_CASE(15) LN_CASE(16) LN_CASE(17) LN_CASE(18) LN_CASE(19) LN_CASE(20) LN_CASE(21)
     LN_CASE(22) LN_CASE(23) LN_CASE(24) LN_CASE(25) LN_CASE(26) LN_CASE(27) LN_CASE(28) LN_CASE(29) LN_CASE(30) LN_CASE(31)
