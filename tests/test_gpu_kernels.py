@@ -239,3 +239,20 @@ def test_cached_filter_spectra_follow_the_weights(gpu):
     mix.cache_filters = False
     y4, _ = mix(u)
     assert torch.equal(y3, y4)
+
+
+def test_encoder_overlapped_filter_generation_matches_sequential(gpu):
+    """Generating layer i + 1's filter spectra on a second stream while layer i runs must not change a bit."""
+    import m2_amd
+    cfg = m2_amd.m2_bert_80m(256)
+    cfg.num_hidden_layers = 3
+    model = m2_amd.BertModel(cfg)
+    model.load_state_dict(m2_amd.seeded_state_dict(cfg, 43))
+    model = model.to(gpu).eval()
+    ids = torch.randint(0, cfg.vocab_size, (2, 256), generator=torch.Generator().manual_seed(10)).to(gpu)
+    want, _ = model(ids)
+    model.encoder.overlap_filters = True
+    for _ in range(3):
+        got, _ = model(ids)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
