@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM-side bytes per mixer-core launch at the default workload, from the two rocprofv3 --pmc runs
 # (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000 against a plain 256 MiB copy); summary in
 # profiles/mixer_core_L8192_B4_hbm_traffic.md.  Only valid for --config c3.
-MIXER_CORE_TRAFFIC_BYTES_C3 = int((212064 * 2.0 + 58368 * 1.0) * 1024)
+MIXER_CORE_TRAFFIC_BYTES_C3 = int((193569 * 2.0 + 68169 * 1.0) * 1024)
 
 
 def workload(name: str):
@@ -236,7 +236,7 @@ def main():
                    "launch": "one captured HIP graph per forward" if args.hip_graph else "eager launches",
                    "eager_ms_per_step": eager_ms,
                    "ms_per_step_with_cached_filter_spectra": cached_ms},
-        "roofline": {"kernel": "mixer_core_kernel (short conv + gates + two FFT long convs + add)",
+        "roofline": {"kernel": "mixer_split_kernel (short conv + gates + two FFT long convs + add)",
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MIXER_CORE_TRAFFIC_BYTES_C3 if args.config == "c3" else None,
