@@ -35,7 +35,7 @@ __device__ __forceinline__ bf16x8 ld8(const uint16_t* p) {
 // fraction of the bf16 rounding the caller applies -- and it costs 12 VALU instructions and no
 // transcendental, where libm erff cost more vector ALU time than the GEMM cost MFMA time.
 __device__ __forceinline__ float gelu_erf(float x) {
-  const float xc = fminf(fmaxf(x, -4.2f), 4.2f);
+  const float xc = __builtin_amdgcn_fmed3f(x, -4.2f, 4.2f);
   const float x2 = xc * xc;
   float p = 5.7684985601e-11f;
   p = fmaf(p, x2, -5.4613545547e-09f);
@@ -353,12 +353,13 @@ __global__ __launch_bounds__(512) void layernorm_kernel(const float* __restrict_
 // Weight-stationary GLU kernel for short K (p = in_features / nblocks <= 256).
 //
 // With K = p as small as 192 a tiled GEMM spends its time filling and draining tiles.  Here a
-// workgroup owns 128 output columns for a long run of rows: wave (mat, ch) keeps the weights of 64
-// columns of ONE of the two GEMMs (mat 0 = gate, 1 = value; ch = which 64 of the 128 columns) in
-// registers for the whole run (KS x 2 MFMA B operands) and the workgroup streams 32-row slabs of x
-// through a single LDS buffer (next slab prefetched into registers during the MFMAs).  Gate and value
-// accumulators meet in an LDS staging tile, where all 256 threads apply gelu(gate) * value and write
-// full 256-byte row segments.  Two barriers per slab.
+// workgroup owns 128 output columns for a long run of rows: wave w keeps, for its 32 columns, the weight
+// rows of BOTH GEMMs (gate block and value block) in registers for the whole run (2 x KS MFMA B
+// operands), so the gate and the value of an output element meet in the same lane and gelu(gate) * value
+// is applied on the accumulators.  The workgroup streams 32-row slabs of x (the K ranges of the two
+// blocks) through a double-buffered LDS tile (the slab after next is in flight in registers during the
+// MFMAs) and the bf16 results go through a small double-buffered LDS tile so that every global store is a
+// full 256-byte row segment, written while the next slab is being multiplied.  One barrier per slab.
 // ---------------------------------------------------------------------------------------------
 template <int KS>        // K steps of 16: p = 16 KS
 __global__ __launch_bounds__(256) void blockdiag_glu_ws_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
@@ -366,15 +367,15 @@ __global__ __launch_bounds__(256) void blockdiag_glu_ws_kernel(const uint16_t* _
                                                                int rows_per_wg) {
   constexpr int p = 16 * KS;
   constexpr int AROW = p + 8;                       // padded bf16 row of an A slab
-  constexpr int SROW = 128 + 4;                     // padded fp32 row of the staging tiles
+  constexpr int GROW = 128 + 8;                     // padded bf16 row of the result tile
   constexpr int CPR = 2 * (p / 8);                  // 16-byte chunks per slab row (gate K-range then value K-range)
   constexpr int NCH = 32 * CPR / 256;               // chunks per thread per slab
+  constexpr int ABUF = 2 * 32 * AROW;               // bf16 elements of one A buffer
   static_assert((32 * CPR) % 256 == 0, "slab must divide over 256 threads");
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  uint16_t* sA = smem;                                                  // [2][32][AROW]
-  float* sS = reinterpret_cast<float*>(smem + 2 * 32 * AROW);           // [2][32][SROW]
+  uint16_t* sA = smem;                              // [2][2][32][AROW]
+  uint16_t* sG = smem + 2 * ABUF;                   // [2][32][GROW]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
-  const int mat = wave >> 1, ch = wave & 1;
   const int I = nb * q / 2, in_f = nb * p;
   const int nslices = I / 128;
   // XCD-aware order: XCD e takes row chunks e, e+8, ... and walks all column slices of one chunk back to back
@@ -391,14 +392,15 @@ __global__ __launch_bounds__(256) void blockdiag_glu_ws_kernel(const uint16_t* _
   const int m_begin = chunk * rows_per_wg;
   const int m_end = min(M, m_begin + rows_per_wg);
 
-  // stationary B operands: rows (blk + mat nb/2, jj + 64 ch + 32 n + i32), K = 16 ks + 8 half + {0..7}
-  bf16x8 bw[2][KS];
+  // stationary B operands: weight rows jj + 32 wave + i32 of block blk (gate) and blk + nb/2 (value),
+  // K = 16 ks + 8 half + {0..7}
+  bf16x8 bwg[KS], bwv[KS];
   {
-    const uint16_t* wp = w + ((long)(blk + mat * (nb / 2)) * q + jj + 64 * ch + i32) * p + 8 * half;
-    static_for<0, 2>([&](auto nn) {
-      static_for<0, KS>([&](auto kk) {
-        bw[decltype(nn)::value][decltype(kk)::value] = ld8(wp + (long)32 * decltype(nn)::value * p + 16 * decltype(kk)::value);
-      });
+    const uint16_t* wg = w + ((long)blk * q + jj + 32 * wave + i32) * p + 8 * half;
+    const uint16_t* wv = wg + (long)(nb / 2) * q * p;
+    static_for<0, KS>([&](auto kk) {
+      bwg[decltype(kk)::value] = ld8(wg + 16 * decltype(kk)::value);
+      bwv[decltype(kk)::value] = ld8(wv + 16 * decltype(kk)::value);
     });
   }
   // per-thread chunk coordinates inside a slab
@@ -419,64 +421,68 @@ __global__ __launch_bounds__(256) void blockdiag_glu_ws_kernel(const uint16_t* _
       ra[j] = *reinterpret_cast<const u32x4*>(x + (long)row * in_f + ccol[j]);
     });
   };
-  auto sstore = [&]() __attribute__((always_inline)) {
-    static_for<0, NCH>([&](auto jj_) { *reinterpret_cast<u32x4*>(sA + clds[decltype(jj_)::value]) = ra[decltype(jj_)::value]; });
+  auto sstore = [&](int buf) __attribute__((always_inline)) {
+    static_for<0, NCH>([&](auto jj_) {
+      *reinterpret_cast<u32x4*>(sA + buf * ABUF + clds[decltype(jj_)::value]) = ra[decltype(jj_)::value];
+    });
+  };
+  // result tile -> global: 32 rows x 256 bytes, two 16-byte pieces per thread
+  auto store_tile = [&](int buf, int m0) __attribute__((always_inline)) {
+    static_for<0, 2>([&](auto jj_) {
+      const int id = tid + 256 * decltype(jj_)::value, r = id >> 4, c = id & 15;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(sG + (buf * 32 + r) * GROW + 8 * c);
+      if (m0 + r < M) *reinterpret_cast<u32x4*>(out + (long)(m0 + r) * I + n0 + 8 * c) = v;
+    });
   };
 
   gload(m_begin);
-  sstore();
-  __syncthreads();
-  const uint16_t* aop = sA + (mat * 32 + i32) * AROW + 8 * half;
-  float* sw_ = sS + mat * 32 * SROW + (4 * half) * SROW + 64 * ch + i32;
-  const int er = tid >> 5, ec = (tid & 31) * 4;                 // epilogue: rows er + 8 it, columns ec .. ec + 3
-  for (int m0 = m_begin; m0 < m_end; m0 += 32) {
-    const bool more = m0 + 32 < m_end;
-    if (more) gload(m0 + 32);
-    floatx16 acc[2];
-    static_for<0, 2>([&](auto nn) { static_for<0, 16>([&](auto vv) { acc[decltype(nn)::value][decltype(vv)::value] = 0.f; }); });
+  sstore(0);
+  if (m_begin + 32 < m_end) gload(m_begin + 32);
+  int s = 0;
+  for (int m0 = m_begin; m0 < m_end; m0 += 32, ++s) {
+    __syncthreads();      // slab s is in sA[s & 1]; result tile s - 1 is complete; buffers of s - 1 are free
+    if (s > 0) store_tile((s - 1) & 1, m0 - 32);
+    const uint16_t* ag = sA + (s & 1) * ABUF + i32 * AROW + 8 * half;
+    const uint16_t* av = ag + 32 * AROW;
+    floatx16 accg, accv;
+    static_for<0, 16>([&](auto vv) { accg[decltype(vv)::value] = 0.f; accv[decltype(vv)::value] = 0.f; });
     static_for<0, KS>([&](auto kk) {
       constexpr int ks = decltype(kk)::value;
-      const bf16x8 a = ld8(aop + 16 * ks);
-      acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bw[0][ks], acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bw[1][ks], acc[1], 0, 0, 0);
+      accg = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(ag + 16 * ks), bwg[ks], accg, 0, 0, 0);
+      accv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(av + 16 * ks), bwv[ks], accv, 0, 0, 0);
     });
-    // accumulator element v: row 8 (v / 4) + 4 half + v % 4, column 32 n + i32 of this wave's 64
-    static_for<0, 2>([&](auto nn) {
-      constexpr int n = decltype(nn)::value;
-      static_for<0, 16>([&](auto vv) {
-        constexpr int v = decltype(vv)::value;
-        sw_[(8 * (v >> 2) + (v & 3)) * SROW + 32 * n] = acc[n][v];
-      });
+    if (m0 + 32 < m_end) {
+      sstore((s + 1) & 1);                     // that buffer was last read before this slab's barrier
+      if (m0 + 64 < m_end) gload(m0 + 64);
+    }
+    // accumulator element v: row 8 (v / 4) + 4 half + v % 4, column 32 wave + i32
+    uint16_t* gt = sG + ((s & 1) * 32 + 4 * half) * GROW + 32 * wave + i32;
+    static_for<0, 8>([&](auto vv) {
+      constexpr int v = 2 * decltype(vv)::value;
+      const uint32_t pk = pack_bf16x2(gelu_erf(accg[v]) * accv[v], gelu_erf(accg[v + 1]) * accv[v + 1]);
+      gt[(8 * (v >> 2) + (v & 3)) * GROW] = (uint16_t)pk;
+      gt[(8 * (v >> 2) + (v & 3) + 1) * GROW] = (uint16_t)(pk >> 16);
     });
-    __syncthreads();                      // staging complete; every wave is done reading the A slab
-    if (more) sstore();
-    static_for<0, 4>([&](auto it_) {
-      constexpr int it = decltype(it_)::value;
-      const int r = er + 8 * it;
-      const int row = m0 + r;
-      const float4 g = *reinterpret_cast<const float4*>(sS + r * SROW + ec);
-      const float4 v = *reinterpret_cast<const float4*>(sS + (32 + r) * SROW + ec);
-      if (row < M) {
-        uint2 pk;
-        pk.x = pack_bf16x2(gelu_erf(g.x) * v.x, gelu_erf(g.y) * v.y);
-        pk.y = pack_bf16x2(gelu_erf(g.z) * v.z, gelu_erf(g.w) * v.w);
-        *reinterpret_cast<uint2*>(out + (long)row * I + n0 + ec) = pk;
-      }
-    });
-    __syncthreads();                      // next slab visible; staging free again
   }
+  __syncthreads();
+  store_tile((s - 1) & 1, m_begin + 32 * (s - 1));
 }
 
 template <int KS>
 static int launch_glu_ws(const void* x, const void* w, void* out, int M, int nb, int q, hipStream_t stream) {
   constexpr int p = 16 * KS;
-  const size_t lds = (size_t)2 * 32 * (p + 8) * sizeof(uint16_t) + (size_t)2 * 32 * 132 * sizeof(float);
+  const size_t lds = ((size_t)2 * 2 * 32 * (p + 8) + (size_t)2 * 32 * (128 + 8)) * sizeof(uint16_t);
+  auto kern = blockdiag_glu_ws_kernel<KS>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(blockdiag_glu_ws): %s", hipGetErrorString(e));
+  }
   const int I = nb * q / 2, nslices = I / 128;
   // rows per workgroup: long runs amortise the weight load, but keep at least ~4 workgroups per CU
   int rows = 512;
   while (rows > 128 && (long)nslices * ((M + rows - 1) / rows) < 4L * num_cus()) rows >>= 1;
   const int nchunks = (M + rows - 1) / rows;
-  hipLaunchKernelGGL(blockdiag_glu_ws_kernel<KS>, dim3(nslices * nchunks), dim3(256), lds, stream, (const uint16_t*)x,
+  hipLaunchKernelGGL(kern, dim3(nslices * nchunks), dim3(256), lds, stream, (const uint16_t*)x,
                      (const uint16_t*)w, (uint16_t*)out, M, nb, q, rows);
   return check_launch("blockdiag_glu_ws");
 }

@@ -15,7 +15,8 @@ int check_launch(const char* what);
 int num_cus();
 
 // round-to-nearest-even float -> bfloat16 bits (NaN stays NaN)
-__host__ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+// float -> bf16 bits, round to nearest even (host restatement of what v_cvt_pk_bf16_f32 does)
+__host__ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
   union { float f; uint32_t u; } v;
   v.f = f;
   if ((v.u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((v.u >> 16) | 0x40u);
@@ -36,7 +37,14 @@ __host__ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   f32x2 v = {lo, hi};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 #else
-  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+#endif
+}
+__host__ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return (uint16_t)pack_bf16x2(f, 0.f);            // the hardware conversion: no branches
+#else
+  return f32_to_bf16_bits(f);
 #endif
 }
 
