@@ -316,9 +316,38 @@ class BertModel(nn.Module):
                 **kwargs):
         if masked_tokens_mask is not None:
             raise NotImplementedError("masked_tokens_mask subsetting belongs to the MLM head, which is not built")
-        # the embedding LayerNorm writes the bf16 and channel-major forms the first layer reads itself
         B, L = input_ids.shape
-        _, h16, hT = self.embeddings.forward_forms(input_ids, token_type_ids, position_ids, want_f32=False)
-        run = self.encoder._run_graphed if self.encoder.use_hip_graph else self.encoder._run_layers
-        enc = [o.view(B, L, -1) for o in run(None, B, L, bool(output_all_encoded_layers), h16=h16, hT=hT)]
+        all_layers = bool(output_all_encoded_layers)
+
+        def run(ids, tt, pos):
+            # the embedding LayerNorm writes the bf16 and channel-major forms the first layer reads itself
+            _, h16, hT = self.embeddings.forward_forms(ids, tt, pos, want_f32=False)
+            return self.encoder._run_layers(None, B, L, all_layers, h16=h16, hT=hT)
+
+        if not self.encoder.use_hip_graph:
+            outs = run(input_ids, token_type_ids, position_ids)
+        else:
+            # embeddings and layer stack as one captured graph per input shape; only the index tensors are copied in
+            given = (input_ids, token_type_ids, position_ids)
+            key = ("model", B, L, all_layers, input_ids.device) + tuple(None if t is None else tuple(t.shape) for t in given)
+            entry = self.encoder._graphs.get(key)
+            if entry is None:
+                static = [None if t is None else t.clone() for t in given]
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):              # warm-up outside the capture (allocator, lazy inits)
+                    run(*static)
+                torch.cuda.current_stream().wait_stream(side)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    static_out = run(*static)
+                entry = (graph, static, static_out)
+                self.encoder._graphs[key] = entry
+            graph, static, static_out = entry
+            for dst, src in zip(static, given):
+                if dst is not None:
+                    dst.copy_(src)
+            graph.replay()
+            outs = [o.clone() for o in static_out]
+        enc = [o.view(B, L, -1) for o in outs]
         return (enc if output_all_encoded_layers else enc[-1]), None
