@@ -141,6 +141,17 @@ int m2_blockdiag_linear_fwd(const void* x, const void* w, const float* bias, con
 int m2_layernorm_fwd(const float* x, const float* gamma, const float* beta, float eps, float* out_f32, void* out_bf16,
                      float* out_channel_major, int M, int d, void* stream);
 
+/* Embedding sum + LayerNorm in one pass (BertEmbeddings.forward in eval mode, bert/src/bert_layers.py:191-252):
+ * row m = b L + l:  e = word_emb[input_ids[m]] + type_emb[token_type_ids[m]] (+ pos_emb[position_ids[m]]),
+ * out = LayerNorm(e) in the same three forms as m2_layernorm_fwd (any may be NULL).
+ * input_ids (B, L) int64; token_type_ids (B, L) int64 or NULL (all zero); pos_emb NULL when the model has no
+ * position embeddings, else position_ids (B, L) int64 or NULL (positions 0 .. L-1 in every sequence).
+ * Tables are fp32 row-major (rows, d); indices are not range-checked.  Needs d % 64 == 0, d <= 2048. */
+int m2_embed_layernorm_fwd(const long long* input_ids, const long long* token_type_ids, const long long* position_ids,
+                           const float* word_emb, const float* type_emb, const float* pos_emb, const float* gamma,
+                           const float* beta, float eps, float* out_f32, void* out_bf16, float* out_channel_major,
+                           int B, int L, int d, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

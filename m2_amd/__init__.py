@@ -1,6 +1,6 @@
 """m2_amd: MI355X (gfx950) kernels for the forward hot path of M2-BERT's Monarch Mixer, behind the
 reference's PyTorch module surface.  Importing the package loads libm2_amd.so and fails if it has
-not been built (`python -m m2_amd.build`); nothing here runs on the CPU."""
+not been built (`python m2_amd/build.py`); nothing here runs on the CPU."""
 from .config import M2BertConfig, m2_bert_80m, m2_bert_large
 from .init import seeded_state_dict
 from . import ops

@@ -27,7 +27,7 @@ class HyenaFilterParams(ctypes.Structure):
 def _load() -> ctypes.CDLL:
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            f"{LIB_PATH} is missing: build it with `python -m m2_amd.build` (hipcc, gfx950). "
+            f"{LIB_PATH} is missing: build it with `python m2_amd/build.py` (hipcc, gfx950). "
             "m2_amd has no CPU or PyTorch fallback for its kernels.")
     lib = ctypes.CDLL(LIB_PATH)
     lib.m2_version.restype = c_int
@@ -56,6 +56,8 @@ def _load() -> ctypes.CDLL:
     lib.m2_layernorm_fwd.restype = c_int
     lib.m2_layernorm_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                      c_void_p]
+    lib.m2_embed_layernorm_fwd.restype = c_int
+    lib.m2_embed_layernorm_fwd.argtypes = [c_void_p] * 8 + [c_float] + [c_void_p] * 3 + [c_int, c_int, c_int, c_void_p]
     return lib
 
 
@@ -63,7 +65,8 @@ lib = _load()
 
 EXPORTS = ["m2_version", "m2_last_error", "m2_hyena_filter_workspace_bytes", "m2_hyena_filter_fwd",
            "m2_fftconv_supported_seqlen", "m2_filter_spectrum_bytes", "m2_filter_spectrum_fwd", "m2_mixer_core_fwd",
-           "m2_fftconv_fwd", "m2_blockdiag_glu_fwd", "m2_blockdiag_linear_fwd", "m2_layernorm_fwd"]
+           "m2_fftconv_fwd", "m2_blockdiag_glu_fwd", "m2_blockdiag_linear_fwd", "m2_layernorm_fwd",
+           "m2_embed_layernorm_fwd"]
 
 
 def check(rc: int) -> None:

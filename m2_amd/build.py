@@ -1,6 +1,6 @@
 """Builds libm2_amd.so (gfx950) from m2_amd/csrc with hipcc, in-tree.
 
-    python -m m2_amd.build            # compile every .hip and link
+    python m2_amd/build.py            # compile every .hip and link
 """
 from __future__ import annotations
 

@@ -263,8 +263,20 @@ struct LnShape {
   static constexpr int PITCH = 64 * PC + 2;
   static constexpr size_t LDS_BYTES = (size_t)R * PITCH * sizeof(float);
 };
-template <int PER>
-__global__ __launch_bounds__(512) void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+// Where the rows come from when the kernel normalises embeddings instead of a matrix:
+// row m = word[ids[m]] + type[tt[m] or 0] (+ pos[pos_ids[m] or m % L]).
+struct EmbedSource {
+  const long long* ids;     // (M)
+  const long long* tt;      // (M) or null: type 0
+  const long long* pos_ids; // (M) or null: m % L
+  const float* word;        // (vocab, d)
+  const float* type;        // (type_vocab, d)
+  const float* pos;         // (max_positions, d) or null: no position embeddings
+  int L;
+};
+template <int PER, bool EMBED>
+__global__ __launch_bounds__(512) void layernorm_kernel(const float* __restrict__ x, EmbedSource src,
+                                                        const float* __restrict__ gamma,
                                                         const float* __restrict__ beta, float eps,
                                                         float* __restrict__ out_f32,       // (M, d) or null
                                                         uint16_t* __restrict__ out_bf16,   // (M, d) or null
@@ -286,8 +298,24 @@ __global__ __launch_bounds__(512) void layernorm_kernel(const float* __restrict_
     constexpr int rr = decltype(rr_)::value;
     int m = m0 + wave * RW + rr;
     m = m < M ? m : M - 1;
-    const float* xr = x + (long)m * d;
-    static_for<0, PER>([&](auto ii) { v[rr][decltype(ii)::value] = xr[lane + 64 * decltype(ii)::value]; });
+    if constexpr (!EMBED) {
+      const float* xr = x + (long)m * d;
+      static_for<0, PER>([&](auto ii) { v[rr][decltype(ii)::value] = xr[lane + 64 * decltype(ii)::value]; });
+    } else {
+      const float* wr = src.word + src.ids[m] * d;
+      const float* tr = src.type + (src.tt ? src.tt[m] : 0) * d;
+      static_for<0, PER>([&](auto ii) {
+        constexpr int i = decltype(ii)::value;
+        v[rr][i] = wr[lane + 64 * i] + tr[lane + 64 * i];
+      });
+      if (src.pos) {
+        const float* pr = src.pos + (src.pos_ids ? src.pos_ids[m] : (long long)(m % src.L)) * d;
+        static_for<0, PER>([&](auto ii) {
+          constexpr int i = decltype(ii)::value;
+          v[rr][i] += pr[lane + 64 * i];
+        });
+      }
+    }
   });
   static_for<0, RW>([&](auto rr_) {
     constexpr int rr = decltype(rr_)::value;
@@ -544,24 +572,22 @@ extern "C" int m2_blockdiag_linear_fwd(const void* x, const void* w, const float
               : launch_blockdiag<4, 1, false, uint16_t, 1>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st);
 }
 
-extern "C" int m2_layernorm_fwd(const float* x, const float* gamma, const float* beta, float eps, float* out_f32,
-                                void* out_bf16, float* out_channel_major, int M, int d, void* stream) {
-  if (!x || !gamma || !beta) return set_error(M2_ERR_ARG, "m2_layernorm_fwd: null pointer");
-  if (M <= 0 || d <= 0 || d % 64 != 0 || d > 2048)
-    return set_error(M2_ERR_UNSUPPORTED, "m2_layernorm_fwd: need M > 0 and d a multiple of 64 up to 2048 (M=%d d=%d)", M, d);
+template <bool EMBED>
+static int launch_layernorm(const float* x, const EmbedSource& src, const float* gamma, const float* beta, float eps,
+                            float* out_f32, void* out_bf16, float* out_channel_major, int M, int d, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   uint16_t* o16 = (uint16_t*)out_bf16;
   switch (d / 64) {
 #define LN_CASE(P)                                                                                                      \
   case P: {                                                                                                             \
     const size_t lds = out_channel_major ? LnShape<P>::LDS_BYTES : 0;                                                   \
-    auto kern = layernorm_kernel<P>;                                                                                    \
+    auto kern = layernorm_kernel<P, EMBED>;                                                                             \
     if (lds > 64 * 1024) {                                                                                              \
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
       if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(layernorm): %s", hipGetErrorString(e)); \
     }                                                                                                                   \
-    hipLaunchKernelGGL(kern, dim3((M + LnShape<P>::R - 1) / LnShape<P>::R), dim3(512), lds, st, x, gamma, beta, eps,   \
-                       out_f32, o16, out_channel_major, M);                                                             \
+    hipLaunchKernelGGL(kern, dim3((M + LnShape<P>::R - 1) / LnShape<P>::R), dim3(512), lds, st, x, src, gamma, beta,   \
+                       eps, out_f32, o16, out_channel_major, M);                                                        \
     break;                                                                                                              \
   }
     LN_CASE(1) LN_CASE(2) LN_CASE(3) LN_CASE(4) LN_CASE(5) LN_CASE(6) LN_CASE(7) LN_CASE(8) LN_CASE(9) LN_CASE(10) LN_CASE(11)
@@ -571,4 +597,27 @@ extern "C" int m2_layernorm_fwd(const float* x, const float* gamma, const float*
 #undef LN_CASE
   }
   return check_launch("layernorm");
+}
+
+extern "C" int m2_layernorm_fwd(const float* x, const float* gamma, const float* beta, float eps, float* out_f32,
+                                void* out_bf16, float* out_channel_major, int M, int d, void* stream) {
+  if (!x || !gamma || !beta) return set_error(M2_ERR_ARG, "m2_layernorm_fwd: null pointer");
+  if (M <= 0 || d <= 0 || d % 64 != 0 || d > 2048)
+    return set_error(M2_ERR_UNSUPPORTED, "m2_layernorm_fwd: need M > 0 and d a multiple of 64 up to 2048 (M=%d d=%d)", M, d);
+  return launch_layernorm<false>(x, EmbedSource{}, gamma, beta, eps, out_f32, out_bf16, out_channel_major, M, d, stream);
+}
+
+extern "C" int m2_embed_layernorm_fwd(const long long* input_ids, const long long* token_type_ids,
+                                      const long long* position_ids, const float* word_emb, const float* type_emb,
+                                      const float* pos_emb, const float* gamma, const float* beta, float eps,
+                                      float* out_f32, void* out_bf16, float* out_channel_major, int B, int L, int d,
+                                      void* stream) {
+  if (!input_ids || !word_emb || !type_emb || !gamma || !beta)
+    return set_error(M2_ERR_ARG, "m2_embed_layernorm_fwd: null pointer");
+  if (B <= 0 || L <= 0 || d <= 0 || d % 64 != 0 || d > 2048)
+    return set_error(M2_ERR_UNSUPPORTED, "m2_embed_layernorm_fwd: need B, L > 0 and d a multiple of 64 up to 2048 (B=%d L=%d d=%d)", B, L, d);
+  if ((long)B * L > 0x7fffffffL) return set_error(M2_ERR_UNSUPPORTED, "m2_embed_layernorm_fwd: B * L = %ld does not fit an int", (long)B * L);
+  if (position_ids && !pos_emb) return set_error(M2_ERR_ARG, "m2_embed_layernorm_fwd: position_ids without a position table");
+  const EmbedSource src{input_ids, token_type_ids, position_ids, word_emb, type_emb, pos_emb, L};
+  return launch_layernorm<true>(nullptr, src, gamma, beta, eps, out_f32, out_bf16, out_channel_major, B * L, d, stream);
 }

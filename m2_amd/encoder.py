@@ -81,11 +81,25 @@ class BertEmbeddings(nn.Module):
         (B, L, d) fp32 | (B*L, d) bf16 | (d, B*L) fp32; forms not asked for are None."""
         if self.training and self.dropout.p > 0:
             raise NotImplementedError("m2_amd is a forward/inference path: call .eval() first")
-        e = self.summed(input_ids, token_type_ids, position_ids, inputs_embeds, past_key_values_length).float()
-        B, L, d = e.shape
-        o32, o16, oT = ops.layernorm(e.reshape(B * L, d).contiguous(), self.LayerNorm.weight.detach().float(),
-                                     self.LayerNorm.bias.detach().float(), self.LayerNorm.eps, want_f32=want_f32,
-                                     want_bf16=want_bf16, want_channel_major=want_channel_major)
+        gamma, beta = self.LayerNorm.weight.detach().float(), self.LayerNorm.bias.detach().float()
+        tables_f32 = self.word_embeddings.weight.dtype == torch.float32
+        if input_ids is not None and inputs_embeds is None and past_key_values_length == 0 and tables_f32:
+            # gather + sum + LayerNorm as one kernel
+            B, L = input_ids.shape
+            d = self.word_embeddings.weight.shape[1]
+            pos = position_ids
+            if pos is not None:
+                pos = pos.expand(B, L).contiguous()
+            o32, o16, oT = ops.embed_layernorm(
+                input_ids.contiguous(), None if token_type_ids is None else token_type_ids.expand(B, L).contiguous(), pos,
+                self.word_embeddings.weight.detach(), self.token_type_embeddings.weight.detach(),
+                self.position_embeddings.weight.detach() if self.use_positional_encodings else None, gamma, beta,
+                self.LayerNorm.eps, want_f32=want_f32, want_bf16=want_bf16, want_channel_major=want_channel_major)
+        else:
+            e = self.summed(input_ids, token_type_ids, position_ids, inputs_embeds, past_key_values_length).float()
+            B, L, d = e.shape
+            o32, o16, oT = ops.layernorm(e.reshape(B * L, d).contiguous(), gamma, beta, self.LayerNorm.eps,
+                                         want_f32=want_f32, want_bf16=want_bf16, want_channel_major=want_channel_major)
         return (None if o32 is None else o32.view(B, L, d)), o16, oT
 
 

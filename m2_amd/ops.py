@@ -195,3 +195,36 @@ def layernorm(x: Tensor, gamma: Tensor, beta: Tensor, eps: float, want_f32: bool
     check(lib.m2_layernorm_fwd(_ptr(x), _ptr(gamma), _ptr(beta), float(eps), _ptr(o32), _ptr(o16), _ptr(ot), M, d,
                                _stream()))
     return o32, o16, ot
+
+
+def embed_layernorm(input_ids: Tensor, token_type_ids: Optional[Tensor], position_ids: Optional[Tensor], word_emb: Tensor,
+                    type_emb: Tensor, pos_emb: Optional[Tensor], gamma: Tensor, beta: Tensor, eps: float,
+                    want_f32: bool = True, want_bf16: bool = False, want_channel_major: bool = False):
+    """LayerNorm(word_emb[ids] + type_emb[token_type_ids or 0] (+ pos_emb[position_ids or 0..L-1])) for ids (B, L)
+    -> (f32 (B*L, d) | None, bf16 (B*L, d) | None, f32 (d, B*L) | None)."""
+    B, L = input_ids.shape
+    d = word_emb.shape[1]
+    _require(input_ids, "input_ids", torch.int64)
+    _require(word_emb, "word_emb", torch.float32)
+    _require(type_emb, "type_emb", torch.float32, (type_emb.shape[0], d))
+    _require(gamma, "gamma", torch.float32, (d,))
+    _require(beta, "beta", torch.float32, (d,))
+    if token_type_ids is not None:
+        _require(token_type_ids, "token_type_ids", torch.int64, (B, L))
+    if pos_emb is not None:
+        _require(pos_emb, "pos_emb", torch.float32, (pos_emb.shape[0], d))
+        if position_ids is None and pos_emb.shape[0] < L:
+            raise ValueError(f"position table has {pos_emb.shape[0]} rows, sequence length is {L}")
+    if position_ids is not None:
+        if pos_emb is None:
+            raise ValueError("position_ids given but the model has no position embeddings")
+        _require(position_ids, "position_ids", torch.int64, (B, L))
+    M = B * L
+    dev = input_ids.device
+    o32 = torch.empty(M, d, dtype=torch.float32, device=dev) if want_f32 else None
+    o16 = torch.empty(M, d, dtype=torch.bfloat16, device=dev) if want_bf16 else None
+    ot = torch.empty(d, M, dtype=torch.float32, device=dev) if want_channel_major else None
+    check(lib.m2_embed_layernorm_fwd(_ptr(input_ids), _ptr(token_type_ids), _ptr(position_ids), _ptr(word_emb),
+                                     _ptr(type_emb), _ptr(pos_emb), _ptr(gamma), _ptr(beta), float(eps), _ptr(o32),
+                                     _ptr(o16), _ptr(ot), B, L, d, _stream()))
+    return o32, o16, ot

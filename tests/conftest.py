@@ -10,6 +10,8 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    import __graft_entry__
+    __graft_entry__.ensure_built()          # compiles only when the tree holds no library yet
 
 
 def rel_err(got, ref):

@@ -256,3 +256,38 @@ def test_encoder_overlapped_filter_generation_matches_sequential(gpu):
         got, _ = model(ids)
         torch.cuda.synchronize()
         assert torch.equal(got, want)
+
+
+def test_embed_layernorm_matches_oracle(gpu):
+    """Gather + sum + LayerNorm kernel against the oracle's BertEmbeddings, with and without explicit
+    token-type / position ids, and against the unfused path (sum by torch ops, then the LayerNorm kernel)."""
+    import m2_amd
+    from oracle import m2_oracle as orc
+    cfg = m2_amd.m2_bert_80m(128)
+    sd = m2_amd.seeded_state_dict(cfg, 17)
+    emb = m2_amd.BertModel(cfg).embeddings
+    emb.load_state_dict({k[len("embeddings."):]: v for k, v in sd.items() if k.startswith("embeddings.")})
+    emb = emb.to(gpu).eval()
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(0, cfg.vocab_size, (3, 100), generator=g)
+    tt = torch.randint(0, cfg.type_vocab_size, (3, 100), generator=g)
+    for use_tt in (False, True):
+        want = orc.embeddings_forward({k: v.double() for k, v in sd.items()}, "embeddings.", ids, cfg,
+                                      token_type_ids=tt if use_tt else None)
+        o32, o16, oT = emb.forward_forms(ids.to(gpu), tt.to(gpu) if use_tt else None)
+        e, e2 = rel_err(o32, want)
+        assert e < 1e-5 and e2 < 1e-5, (use_tt, e, e2)
+        assert torch.equal(oT, o32.reshape(-1, o32.shape[-1]).t())
+        assert torch.equal(o16, o32.reshape(-1, o32.shape[-1]).to(torch.bfloat16))
+        # unfused path: explicit inputs_embeds
+        o32b, _, _ = emb.forward_forms(None, tt.to(gpu) if use_tt else None, None,
+                                       inputs_embeds=emb.word_embeddings(ids.to(gpu)), want_bf16=False, want_channel_major=False)
+        assert (o32b - o32).abs().max().item() < 1e-5
+    if cfg.use_positional_encodings:
+        pos = torch.arange(100).flip(0)[None]
+        o32, _, _ = emb.forward_forms(ids.to(gpu), None, pos.to(gpu), want_bf16=False, want_channel_major=False)
+        e = emb.summed(ids.to(gpu), None, pos.to(gpu)).double().cpu()
+        want = torch.nn.functional.layer_norm(e, (e.shape[-1],), sd["embeddings.LayerNorm.weight"].double(),
+                                              sd["embeddings.LayerNorm.bias"].double(), cfg.layer_norm_eps)
+        err, err2 = rel_err(o32, want)
+        assert err < 1e-5 and err2 < 1e-5
