@@ -157,14 +157,17 @@ class BertLayer(nn.Module):
             a, _ = self.attention(hidden_states)
         return self.mlp(a)
 
-    def fused(self, h16: torch.Tensor, hT: Optional[torch.Tensor], B: int, L: int, want_f32: bool,
-              spec: Optional[torch.Tensor] = None, spec_ready=None, after_core=None):
+    def fused(self, h16: Optional[torch.Tensor], hT: Optional[torch.Tensor], B: int, L: int, want_f32: bool,
+              spec: Optional[torch.Tensor] = None, spec_ready=None, after_core=None,
+              h32: Optional[torch.Tensor] = None):
         """One layer of the fused schedule.  h16 (M,d) bf16, hT (d,M) f32 -> (f32 | None, bf16, (d,M) f32).
         `spec`: this layer's filter spectra when the caller has generated them already (`spec_ready`: the event
         the current stream must wait for before reading them); `after_core()` is called once the mixer core
         has been enqueued."""
         at = self.attention
         d = at.d_model
+        if at.hyena_training_additions:      # extra input LayerNorm: needs the fp32 form, replaces h16 / hT
+            _, h16, hT = at.pre_norm(h32, want_f32=False, want_bf16=True)
         w_in = at._cast("in_w", at.in_linear.weight, torch.bfloat16)
         w_out = at._cast("out_w", at.out_linear.weight, torch.bfloat16)
         b_out = at._cast("out_b", at.out_linear.bias, torch.bfloat16)
@@ -177,7 +180,8 @@ class BertLayer(nn.Module):
         a16 = torch.addmm(b_out, y.view(d, B * L).t(), w_out.t())                    # (M, d)
         s = self.mlp.presum(a16)
         gamma, beta, eps = self.mlp.ln_params()
-        return ops.layernorm(s, gamma, beta, eps, want_f32=want_f32, want_bf16=True, want_channel_major=True)
+        pre = at.hyena_training_additions        # the next layer then reads the fp32 form only
+        return ops.layernorm(s, gamma, beta, eps, want_f32=want_f32, want_bf16=not pre, want_channel_major=not pre)
 
 
 class BertEncoder(nn.Module):
@@ -220,10 +224,12 @@ class BertEncoder(nn.Module):
         that already holds the bf16 and the channel-major fp32 form of the input passes them as h16 / hT (and
         may then pass h32 = None)."""
         with torch.autocast("cuda", enabled=False):
-            if h16 is None:
-                h16 = h32.to(torch.bfloat16)
-            if hT is None:
-                hT = h32.t().contiguous()
+            pre_norm = self.layer[0].attention.hyena_training_additions       # layers then start from the fp32 form
+            if not pre_norm:
+                if h16 is None:
+                    h16 = h32.to(torch.bfloat16)
+                if hT is None:
+                    hT = h32.t().contiguous()
             outs = []
             n = len(self.layer)
             o32 = h32
@@ -250,6 +256,7 @@ class BertEncoder(nn.Module):
                 generate(0, None)
             for i, layer in enumerate(self.layer):
                 want = all_layers or i == n - 1
+                keep32 = want or pre_norm
                 spec, ready, hook = None, None, None
                 if overlap:
                     spec, ready = nxt
@@ -258,7 +265,8 @@ class BertEncoder(nn.Module):
                             ev = torch.cuda.Event()
                             ev.record(cur)
                             generate(i + 1, ev)
-                o32, h16, hT = layer.fused(h16, hT, B, L, want_f32=want, spec=spec, spec_ready=ready, after_core=hook)
+                o32, h16, hT = layer.fused(h16, hT, B, L, want_f32=keep32, spec=spec, spec_ready=ready,
+                                           after_core=hook, h32=o32)
                 if want:
                     outs.append(o32)
             if overlap:
@@ -333,10 +341,15 @@ class BertModel(nn.Module):
         B, L = input_ids.shape
         all_layers = bool(output_all_encoded_layers)
 
+        pre_norm = self.encoder.layer[0].attention.hyena_training_additions
+
         def run(ids, tt, pos):
             # the embedding LayerNorm writes the bf16 and channel-major forms the first layer reads itself
-            _, h16, hT = self.embeddings.forward_forms(ids, tt, pos, want_f32=False)
-            return self.encoder._run_layers(None, B, L, all_layers, h16=h16, hT=hT)
+            # (or the fp32 form when the layers start with their own LayerNorm)
+            h32, h16, hT = self.embeddings.forward_forms(ids, tt, pos, want_f32=pre_norm, want_bf16=not pre_norm,
+                                                         want_channel_major=not pre_norm)
+            return self.encoder._run_layers(None if h32 is None else h32.view(B * L, -1), B, L, all_layers,
+                                            h16=h16, hT=hT)
 
         if not self.encoder.use_hip_graph:
             outs = run(input_ids, token_type_ids, position_ids)

@@ -70,6 +70,9 @@ def mixer_state(prefix: str, cfg: M2BertConfig, gen, std: float) -> Dict[str, to
     sd[prefix + "out_linear.bias"] = torch.zeros(d)
     sd[prefix + "short_filter.weight"] = _normal(gen, 3 * d, 1, 3, std=std)
     sd[prefix + "short_filter.bias"] = torch.zeros(3 * d)
+    if cfg.hyena_training_additions:       # the extra pre-LayerNorm (monarch_mixer_sequence_mixer.py:84-87)
+        sd[prefix + "layernorm.weight"] = torch.ones(d) + _normal(gen, d, std=std)
+        sd[prefix + "layernorm.bias"] = _normal(gen, d, std=std)
     return sd
 
 

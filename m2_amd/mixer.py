@@ -29,8 +29,6 @@ class MonarchMixerSequenceMixing(nn.Module):
                  hyena_filter_dropout=0.0, hyena_filter_order=16, residual_long_conv=False,
                  hyena_training_additions=False):
         super().__init__()
-        if hyena_training_additions:
-            raise NotImplementedError("hyena_training_additions=True (extra LayerNorm/dropout) is not built")
         self.d_model = d_model
         self.l_max = l_max
         self.kernel_lr = hyena_kernel_lr
@@ -50,6 +48,12 @@ class MonarchMixerSequenceMixing(nn.Module):
             self.filter_fn2 = make_filter()
         self.in_linear = nn.Linear(d_model, 3 * d_model)
         self.out_linear = nn.Linear(d_model, d_model)
+        if self.hyena_training_additions:
+            # extra pre-LayerNorm; the dropouts and the Identity activation do nothing in a forward-only path
+            # (bert/src/mm/monarch_mixer_sequence_mixer.py:84-87,102-103,118-119,150-151)
+            self.act = nn.Identity()
+            self.drop = nn.Dropout(dropout)
+            self.layernorm = nn.LayerNorm(d_model)
         total_width = self.d_model * self.NUM_PROJECTIONS
         self.short_filter = nn.Conv1d(in_channels=total_width, out_channels=total_width, kernel_size=3,
                                       groups=total_width, padding=2)
@@ -106,6 +110,13 @@ class MonarchMixerSequenceMixing(nn.Module):
         pb = self._cast("in_b32", self.in_linear.bias, torch.float32)
         return ops.mixer_core(xproj, u_cm, sw, sb, spec, B, L, self.d_model, proj_bias=pb)
 
+    def pre_norm(self, h32: torch.Tensor, want_f32: bool, want_bf16: bool):
+        """The extra input LayerNorm of hyena_training_additions: (M, d) fp32 -> (f32 | None, bf16 | None,
+        channel-major f32 (d, M) | None when there is no residual long convolution)."""
+        ln = self.layernorm
+        return ops.layernorm(h32, ln.weight.detach().float(), ln.bias.detach().float(), ln.eps, want_f32=want_f32,
+                             want_bf16=want_bf16, want_channel_major=self.residual_long_conv)
+
     # -- reference API -----------------------------------------------------------------------
     def forward(self, u, **kwargs):
         if not u.is_cuda:
@@ -120,8 +131,18 @@ class MonarchMixerSequenceMixing(nn.Module):
         w_out = self._cast("out_w", self.out_linear.weight, act)
         b_out = self._cast("out_b", self.out_linear.bias, act)
         with torch.autocast("cuda", enabled=False):
+            u_cm = None
+            if self.hyena_training_additions:
+                if self.training and self.drop.p > 0:
+                    raise NotImplementedError("m2_amd is a forward/inference path: call .eval() first")
+                u2, u16, u_cm = self.pre_norm(u2.float().contiguous(), want_f32=not low, want_bf16=low)
+                if low:
+                    u2 = u16
             xproj = torch.mm(w_in, u2.to(act).t())                                      # (3d, B*L), bias added in the core
-            u_cm = u2.float().t().contiguous() if self.residual_long_conv else None      # (d, B*L)
+            if u_cm is None and self.residual_long_conv:
+                u_cm = u2.float().t().contiguous()                                       # (d, B*L)
+            if not self.residual_long_conv:
+                u_cm = None
             y = self.core(xproj.view(3 * d, B, L), None if u_cm is None else u_cm.view(d, B, L), B, L)
             out = torch.addmm(b_out, y.view(d, B * L).t(), w_out.t())                   # (B*L, d)
         return out.view(B, L, d), None

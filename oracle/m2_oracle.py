@@ -176,13 +176,19 @@ def mixer_filters(sd: StateDict, prefix: str, L: int, bidirectional: bool = True
 
 
 def mixer_forward(sd: StateDict, prefix: str, u: Tensor, bidirectional: bool = True,
-                  residual_long_conv: bool = True, w_mod: float = 1.0, emulate_autocast: bool = False) -> Tensor:
-    """MonarchMixerSequenceMixing.forward, u (B, L, d) -> (B, L, d).
+                  residual_long_conv: bool = True, w_mod: float = 1.0, emulate_autocast: bool = False,
+                  training_additions: bool = False) -> Tensor:
+    """MonarchMixerSequenceMixing.forward in eval mode, u (B, L, d) -> (B, L, d).
 
-    bert/src/mm/monarch_mixer_sequence_mixer.py:100-154 with hyena_training_additions=False.
+    bert/src/mm/monarch_mixer_sequence_mixer.py:100-154.  With hyena_training_additions the input goes through
+    an extra nn.LayerNorm(d_model) (default eps 1e-5, :84-87, :102-103) and that normalised input is also what
+    the residual long convolution sees (:107); the two dropouts and the Identity activation (:118-119,
+    :150-151) do nothing in eval mode.
     """
     B, L, d = u.shape
     rd = _rd(emulate_autocast)
+    if training_additions:
+        u = F.layer_norm(u, (d,), sd[prefix + "layernorm.weight"], sd[prefix + "layernorm.bias"], 1e-5)
     u_orig = u
     x = rd(F.linear(rd(u), rd(sd[prefix + "in_linear.weight"]), rd(sd[prefix + "in_linear.bias"])))
     x = x.transpose(1, 2)                                             # (B, 3d, L)
@@ -253,7 +259,7 @@ def layer_forward(sd: StateDict, prefix: str, x: Tensor, cfg, emulate_autocast: 
     bert/src/bert_layers.py:575-599.
     """
     a = mixer_forward(sd, prefix + "attention.", x, cfg.bidirectional, cfg.residual_long_conv,
-                      cfg.hyena_w_mod, emulate_autocast)
+                      cfg.hyena_w_mod, emulate_autocast, getattr(cfg, "hyena_training_additions", False))
     return glu_mlp_forward(sd, prefix + "mlp.", a, cfg.intermediate_size, cfg.layer_norm_eps, emulate_autocast)
 
 

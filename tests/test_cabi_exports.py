@@ -93,6 +93,13 @@ def test_state_dict_names_match_the_reference_layout():
             expect |= {q + mlp + f"{i}.bias" for i in (0, 2, 4)}
             expect |= {q + mlp + f"{i}.freq" for i in (1, 3, 5)}
     assert keys == expect
+    # hyena_training_additions adds the mixer's own LayerNorm (bert/src/mm/monarch_mixer_sequence_mixer.py:84-87)
+    cfg2 = m2_amd.m2_bert_80m(128)
+    cfg2.num_hidden_layers = 1
+    cfg2.hyena_training_additions = True
+    keys2 = set(m2_amd.BertModel(cfg2).state_dict().keys())
+    assert keys2 == expect | {p + "attention.layernorm.weight", p + "attention.layernorm.bias"}
+    assert set(m2_amd.seeded_state_dict(cfg2, 1).keys()) == keys2
     m = m2_amd.BertModel(cfg)
     sd = m.state_dict()
     assert tuple(sd[p + "attention.short_filter.weight"].shape) == (3 * 768, 1, 3)

@@ -291,3 +291,44 @@ def test_embed_layernorm_matches_oracle(gpu):
                                               sd["embeddings.LayerNorm.bias"].double(), cfg.layer_norm_eps)
         err, err2 = rel_err(o32, want)
         assert err < 1e-5 and err2 < 1e-5
+
+
+def test_mixer_and_encoder_with_training_additions(gpu):
+    """hyena_training_additions=True (the extra input LayerNorm of the mixer): one fp32 mixer at 1e-4, and a
+    two-layer encoder (fused schedule, graph replay, module-by-module path) at the bf16 tolerance."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    cfg = m2_amd.m2_bert_80m(128)
+    cfg.hyena_training_additions = True
+    cfg.num_hidden_layers = 2
+    sdm = m2_amd.seeded_state_dict(cfg, 77, what="mixer")
+    mix = m2_amd.MonarchMixerSequenceMixing(768, l_max=128, bidirectional=True, hyena_emb_dim=5, hyena_filter_order=128,
+                                            residual_long_conv=True, hyena_w=10, hyena_w_mod=1,
+                                            hyena_training_additions=True)
+    mix.load_state_dict(sdm)
+    mix = mix.to(gpu).eval()
+    u = torch.randn(4, 128, 768, generator=torch.Generator().manual_seed(8)) * 2 + 0.5
+    y, _ = mix(u.to(gpu))
+    e, e2 = rel_err(y, O.mixer_forward(sdm, "", u, training_additions=True))
+    assert e < TOL_F32 and e2 < TOL_F32, (e, e2)
+
+    sd = m2_amd.seeded_state_dict(cfg, 78)
+    model = m2_amd.BertModel(cfg)
+    model.load_state_dict(sd)
+    model = model.to(gpu).eval()
+    ids = torch.randint(0, cfg.vocab_size, (3, 128), generator=torch.Generator().manual_seed(6))
+    ref = O.model_forward(sd, ids, None, cfg)
+    out, _ = model(ids.to(gpu))
+    e, e2 = rel_err(out, ref)
+    assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
+    model.encoder.use_hip_graph = True
+    for _ in range(2):
+        got, _ = model(ids.to(gpu))
+        torch.cuda.synchronize()
+        assert torch.equal(got, out)
+    model.encoder.use_hip_graph = False
+    x = model.embeddings(ids.to(gpu))
+    for layer in model.encoder.layer:
+        x = layer(x)
+    e, e2 = rel_err(x, ref)
+    assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)

@@ -350,3 +350,25 @@ def test_autocast_emulation_is_a_small_perturbation_of_fp32():
     b = O.model_forward(sd, ids, None, cfg, emulate_autocast=True)
     rel = ((a - b).norm() / a.norm()).item()
     assert 1e-4 < rel < 2e-2
+
+
+def test_mixer_training_additions_is_a_pre_layernorm_seen_by_both_convolutions():
+    """hyena_training_additions in eval mode: the input LayerNorm (eps 1e-5) feeds the projections AND the
+    residual long convolution (monarch_mixer_sequence_mixer.py:102-107); everything else is unchanged.  Checked
+    by composing the plain mixer with an explicitly computed LayerNorm, and by showing that normalising only the
+    projection input (the plausible mistake) gives a different answer."""
+    import m2_amd
+    cfg = m2_amd.m2_bert_80m(64)
+    cfg.hidden_size = 64
+    cfg.hyena_training_additions = True
+    sd = {k: v.double() for k, v in m2_amd.seeded_state_dict(cfg, 5, std=0.3, what="mixer").items()}
+    u = torch.randn(2, 64, 64, dtype=torch.float64, generator=torch.Generator().manual_seed(2)) * 3 + 1.5
+    got = O.mixer_forward(sd, "", u, True, True, 1.0, False, True)
+    mu = u.mean(-1, keepdim=True)
+    var = ((u - mu) ** 2).mean(-1, keepdim=True)
+    un = (u - mu) / torch.sqrt(var + 1e-5) * sd["layernorm.weight"] + sd["layernorm.bias"]
+    want = O.mixer_forward(sd, "", un, True, True, 1.0, False, False)
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
+    # the residual convolution must see the normalised input: feeding it the raw input changes the result
+    plain = O.mixer_forward(sd, "", u, True, True, 1.0, False, False)
+    assert (got - plain).abs().max() > 1e-3
