@@ -7,8 +7,10 @@ from . import ops
 from .hyena import HyenaFilter, Sin, PositionalEmbedding, ExponentialModulation
 from .mixer import MonarchMixerSequenceMixing
 from .blockdiag import BlockdiagLinear, blockdiag_multiply
-from .encoder import BertEmbeddings, BertGatedLinearUnitMLP, BertLayer, BertEncoder, BertModel
+from .encoder import BertEmbeddings, BertGatedLinearUnitMLP, BertLayer, BertEncoder, BertModel, BertPooler
+from .embed import M2BertTextEncoder
 
 __all__ = ["M2BertConfig", "m2_bert_80m", "m2_bert_large", "seeded_state_dict", "ops", "HyenaFilter", "Sin",
            "PositionalEmbedding", "ExponentialModulation", "MonarchMixerSequenceMixing", "BlockdiagLinear",
-           "blockdiag_multiply", "BertEmbeddings", "BertGatedLinearUnitMLP", "BertLayer", "BertEncoder", "BertModel"]
+           "blockdiag_multiply", "BertEmbeddings", "BertGatedLinearUnitMLP", "BertLayer", "BertEncoder", "BertModel",
+           "BertPooler", "M2BertTextEncoder"]

@@ -48,7 +48,10 @@ class M2BertConfig:
     use_positional_encodings: bool = True
     use_flash_mm: bool = False
     use_flash_fft: bool = False
-    pool_all: bool = False
+    pool_all: bool = False                     # BertPooler: masked mean over the sequence instead of the first token
+    use_cls_token: bool = False                # read by the reference's pooler constructor, not by its forward
+    sequence_token_planting: bool = False
+    attention_pooling: bool = False
 
     def with_seq_len(self, L: int) -> "M2BertConfig":
         return replace(self, max_position_embeddings=L, long_conv_l_max=L)

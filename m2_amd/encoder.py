@@ -317,17 +317,41 @@ class BertEncoder(nn.Module):
         return outs
 
 
-class BertModel(nn.Module):
-    """Embeddings + encoder (no pooler: the heads are outside the accelerated path)."""
+class BertPooler(nn.Module):
+    """tanh(dense(first token)), or with config.pool_all tanh(dense(mean over unmasked positions))
+    (bert/src/bert_layers.py:816-859).  A (B, d) x (d, d) product: plain torch ops."""
 
-    def __init__(self, config: M2BertConfig, add_pooling_layer: bool = False, use_hip_graph: bool = False):
+    def __init__(self, config: M2BertConfig):
         super().__init__()
-        if add_pooling_layer:
-            raise NotImplementedError("pooler / heads are not part of this path")
+        if getattr(config, "sequence_token_planting", False):
+            raise NotImplementedError("sequence_token_planting pooling is not built")
+        self.dense = nn.Linear(config.hidden_size, config.hidden_size)
+        self.activation = nn.Tanh()
+        self.pool_all = getattr(config, "pool_all", False)
+        self.use_cls_token = getattr(config, "use_cls_token", False)
+        self.sequence_token_planting = False
+
+    def forward(self, hidden_states: torch.Tensor, pool: Optional[bool] = True, mask=None) -> torch.Tensor:
+        if not self.pool_all:
+            first = hidden_states[:, 0] if pool else hidden_states
+            return self.activation(self.dense(first))
+        m = mask.to(hidden_states.dtype)
+        mean = torch.sum(hidden_states * m.unsqueeze(-1), dim=1) / torch.sum(m, dim=1, keepdim=True)
+        return self.activation(self.dense(mean))
+
+
+class BertModel(nn.Module):
+    """Embeddings + encoder + pooler; returns (sequence output or list of layer outputs, pooled output or None)
+    like the reference (bert/src/bert_layers.py:880-1010)."""
+
+    def __init__(self, config: M2BertConfig, add_pooling_layer: bool = True, use_hip_graph: bool = False):
+        super().__init__()
+        if getattr(config, "attention_pooling", False):
+            raise NotImplementedError("attention_pooling is not built")
         self.config = config
         self.embeddings = BertEmbeddings(config)
         self.encoder = BertEncoder(config, use_hip_graph=use_hip_graph)
-        self.pooler = None
+        self.pooler = BertPooler(config) if add_pooling_layer else None
 
     def get_input_embeddings(self):
         return self.embeddings.word_embeddings
@@ -377,4 +401,9 @@ class BertModel(nn.Module):
             graph.replay()
             outs = [o.clone() for o in static_out]
         enc = [o.view(B, L, -1) for o in outs]
-        return (enc if output_all_encoded_layers else enc[-1]), None
+        pooled = None
+        if self.pooler is not None:
+            if attention_mask is None:
+                attention_mask = torch.ones_like(input_ids)
+            pooled = self.pooler(enc[-1], mask=attention_mask)
+        return (enc if output_all_encoded_layers else enc[-1]), pooled

@@ -87,8 +87,10 @@ def mlp_state(prefix: str, cfg: M2BertConfig, gen, std: float) -> Dict[str, torc
     }
 
 
-def seeded_state_dict(cfg: M2BertConfig, seed: int, std: float | None = None, what: str = "model") -> Dict[str, torch.Tensor]:
-    """`what`: 'model' (BertModel keys), 'mixer' (one MonarchMixerSequenceMixing), 'mlp' (one GLU MLP)."""
+def seeded_state_dict(cfg: M2BertConfig, seed: int, std: float | None = None, what: str = "model",
+                      pooler: bool = True) -> Dict[str, torch.Tensor]:
+    """`what`: 'model' (BertModel keys, with the pooler's unless pooler=False), 'mixer' (one
+    MonarchMixerSequenceMixing), 'mlp' (one GLU MLP)."""
     gen = torch.Generator().manual_seed(seed)
     std = cfg.initializer_range if std is None else std
     if what == "mixer":
@@ -108,4 +110,7 @@ def seeded_state_dict(cfg: M2BertConfig, seed: int, std: float | None = None, wh
     for i in range(cfg.num_hidden_layers):
         sd.update(mixer_state(f"encoder.layer.{i}.attention.", cfg, gen, std))
         sd.update(mlp_state(f"encoder.layer.{i}.mlp.", cfg, gen, std))
+    if pooler:      # drawn last, so the other tensors do not depend on it
+        sd["pooler.dense.weight"] = _normal(gen, d, d, std=std)
+        sd["pooler.dense.bias"] = _normal(gen, d, std=std)
     return sd

@@ -294,15 +294,32 @@ def embeddings_forward(sd: StateDict, prefix: str, input_ids: Tensor, cfg,
                         cfg.layer_norm_eps)
 
 
-def model_forward(sd: StateDict, input_ids: Tensor, attention_mask: Optional[Tensor], cfg,
-                  prefix: str = "", emulate_autocast: bool = False) -> Tensor:
-    """BertModel.forward without pooler: embeddings -> encoder, last hidden state (B, L, d).
+def pooler_forward(sd: StateDict, prefix: str, hidden: Tensor, mask: Optional[Tensor], pool_all: bool) -> Tensor:
+    """BertPooler.forward (bert/src/bert_layers.py:816-859) without sequence_token_planting:
+    tanh(dense(first token)), or with pool_all tanh(dense(mean over the positions whose mask is 1))."""
+    if not pool_all:
+        pooled = hidden[:, 0]
+    else:
+        m = mask.to(hidden.dtype)
+        pooled = (hidden * m.unsqueeze(-1)).sum(dim=1) / m.sum(dim=1, keepdim=True)
+    return torch.tanh(F.linear(pooled, sd[prefix + "dense.weight"], sd[prefix + "dense.bias"]))
 
-    bert/src/bert_layers.py:948-985.
+
+def model_forward(sd: StateDict, input_ids: Tensor, attention_mask: Optional[Tensor], cfg,
+                  prefix: str = "", emulate_autocast: bool = False, pooled: bool = False):
+    """BertModel.forward: embeddings -> encoder, last hidden state (B, L, d); with pooled=True also the
+    pooler's output, as a pair.
+
+    bert/src/bert_layers.py:948-1010.
     """
     x = embeddings_forward(sd, prefix + "embeddings.", input_ids, cfg)
-    return encoder_forward(sd, prefix + "encoder.", x, attention_mask, cfg,
-                           emulate_autocast=emulate_autocast)[-1]
+    seq = encoder_forward(sd, prefix + "encoder.", x, attention_mask, cfg,
+                          emulate_autocast=emulate_autocast)[-1]
+    if not pooled:
+        return seq
+    if attention_mask is None:
+        attention_mask = torch.ones_like(input_ids)
+    return seq, pooler_forward(sd, prefix + "pooler.", seq, attention_mask, getattr(cfg, "pool_all", False))
 
 
 def cast_state_dict(sd: StateDict, dtype) -> StateDict:

@@ -80,7 +80,7 @@ def test_state_dict_names_match_the_reference_layout():
     p = "encoder.layer.0."
     expect = {"embeddings.word_embeddings.weight", "embeddings.position_embeddings.weight",
               "embeddings.token_type_embeddings.weight", "embeddings.LayerNorm.weight", "embeddings.LayerNorm.bias",
-              "embeddings.position_ids",
+              "embeddings.position_ids", "pooler.dense.weight", "pooler.dense.bias",
               p + "attention.in_linear.weight", p + "attention.in_linear.bias", p + "attention.out_linear.weight",
               p + "attention.out_linear.bias", p + "attention.short_filter.weight", p + "attention.short_filter.bias",
               p + "mlp.gated_layers.weight", p + "mlp.wo.weight", p + "mlp.wo.bias", p + "mlp.layernorm.weight",
@@ -93,6 +93,8 @@ def test_state_dict_names_match_the_reference_layout():
             expect |= {q + mlp + f"{i}.bias" for i in (0, 2, 4)}
             expect |= {q + mlp + f"{i}.freq" for i in (1, 3, 5)}
     assert keys == expect
+    assert set(m2_amd.BertModel(cfg, add_pooling_layer=False).state_dict().keys()) == \
+        expect - {"pooler.dense.weight", "pooler.dense.bias"}
     # hyena_training_additions adds the mixer's own LayerNorm (bert/src/mm/monarch_mixer_sequence_mixer.py:84-87)
     cfg2 = m2_amd.m2_bert_80m(128)
     cfg2.num_hidden_layers = 1

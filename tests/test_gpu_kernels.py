@@ -332,3 +332,44 @@ def test_mixer_and_encoder_with_training_additions(gpu):
         x = layer(x)
     e, e2 = rel_err(x, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
+
+
+@pytest.mark.parametrize("pool_all", [False, True])
+def test_pooled_output_and_text_encoder_loop(gpu, pool_all):
+    """BertModel's pooled output against the oracle, and the embedding caller's batching loop (ragged and empty
+    texts, padding, truncation, last partial batch) against one-at-a-time oracle results."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    cfg = m2_amd.m2_bert_80m(128)
+    cfg.num_hidden_layers = 1
+    cfg.pool_all = pool_all
+    sd = m2_amd.seeded_state_dict(cfg, 61)
+    model = m2_amd.BertModel(cfg)
+    model.load_state_dict(sd)
+    model = model.to(gpu).eval()
+    g = torch.Generator().manual_seed(12)
+    lengths = [5, 128, 0 if not pool_all else 1, 200, 64]       # an empty text has no mean: only with CLS pooling
+    texts = [torch.randint(1, cfg.vocab_size, (n,), generator=g) for n in lengths]
+    enc = m2_amd.M2BertTextEncoder(model, max_seq_len=128)
+    got = enc.encode_token_ids(texts, batch_size=2)
+    assert got.shape == (len(texts), cfg.hidden_size) and got.dtype.name == "float32"
+    for k, ids in enumerate(texts):
+        row = torch.zeros(1, 128, dtype=torch.long)
+        n = min(len(ids), 128)
+        row[0, :n] = ids[:n]
+        mask = torch.zeros(1, 128, dtype=torch.long)
+        mask[0, :n] = 1
+        _, want = O.model_forward(sd, row, mask, cfg, pooled=True)
+        err = (torch.from_numpy(got[k]) - want[0]).abs().max().item()
+        assert err < 2e-2, (k, err)
+
+    class WordTokenizer:                      # stands in for a Hugging Face tokenizer (same calling convention)
+        def __call__(self, batch, return_tensors="pt"):
+            ids = torch.tensor([[101] + [1000 + (hash(w) % 20000) for w in batch[0].split()] + [102]])
+            return {"input_ids": ids, "attention_mask": torch.ones_like(ids)}
+    enc = m2_amd.M2BertTextEncoder(model, max_seq_len=128, tokenizer=WordTokenizer())
+    q = enc.encode_queries(["monarch mixer", "a longer query about sub-quadratic sequence models", "x"], batch_size=2)
+    c = enc.encode_corpus([{"title": "T", "text": "some passage"}, {"title": "U", "text": "another"}], batch_size=8)
+    assert q.shape == (3, cfg.hidden_size) and c.shape == (2, cfg.hidden_size)
+    again = enc.encode_queries(["x"], batch_size=1)
+    assert abs(again[0] - q[2]).max() < 2e-2          # same text alone or inside a batch

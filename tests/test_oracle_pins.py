@@ -372,3 +372,24 @@ def test_mixer_training_additions_is_a_pre_layernorm_seen_by_both_convolutions()
     # the residual convolution must see the normalised input: feeding it the raw input changes the result
     plain = O.mixer_forward(sd, "", u, True, True, 1.0, False, False)
     assert (got - plain).abs().max() > 1e-3
+
+
+def test_pooler_first_token_and_masked_mean():
+    """BertPooler (bert/src/bert_layers.py:816-859): tanh(W h[:, 0] + b), and with pool_all the mean over the
+    positions whose mask is 1 only -- checked against explicit per-example loops."""
+    g = torch.Generator().manual_seed(11)
+    B, L, d = 3, 7, 5
+    h = torch.randn(B, L, d, dtype=torch.float64, generator=g)
+    sd = {"dense.weight": torch.randn(d, d, dtype=torch.float64, generator=g),
+          "dense.bias": torch.randn(d, dtype=torch.float64, generator=g)}
+    mask = torch.tensor([[1, 1, 1, 0, 0, 0, 0], [1, 1, 1, 1, 1, 1, 1], [1, 0, 0, 0, 0, 0, 0]])
+    cls = O.pooler_forward(sd, "", h, mask, pool_all=False)
+    mean = O.pooler_forward(sd, "", h, mask, pool_all=True)
+    for b in range(B):
+        want = torch.tanh(sd["dense.weight"] @ h[b, 0] + sd["dense.bias"])
+        assert torch.allclose(cls[b], want, atol=1e-14)
+        n = int(mask[b].sum())
+        avg = sum(h[b, l] for l in range(L) if mask[b, l] == 1) / n
+        assert torch.allclose(mean[b], torch.tanh(sd["dense.weight"] @ avg + sd["dense.bias"]), atol=1e-14)
+    # one real token: both poolings coincide
+    assert torch.allclose(cls[2], mean[2], atol=1e-14)
