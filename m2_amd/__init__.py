@@ -9,8 +9,9 @@ from .mixer import MonarchMixerSequenceMixing
 from .blockdiag import BlockdiagLinear, blockdiag_multiply
 from .encoder import BertEmbeddings, BertGatedLinearUnitMLP, BertLayer, BertEncoder, BertModel, BertPooler
 from .embed import M2BertTextEncoder
+from .checkpoint import load_reference_checkpoint, extend_context
 
 __all__ = ["M2BertConfig", "m2_bert_80m", "m2_bert_large", "seeded_state_dict", "ops", "HyenaFilter", "Sin",
            "PositionalEmbedding", "ExponentialModulation", "MonarchMixerSequenceMixing", "BlockdiagLinear",
            "blockdiag_multiply", "BertEmbeddings", "BertGatedLinearUnitMLP", "BertLayer", "BertEncoder", "BertModel",
-           "BertPooler", "M2BertTextEncoder"]
+           "BertPooler", "M2BertTextEncoder", "load_reference_checkpoint", "extend_context"]

@@ -373,3 +373,26 @@ def test_pooled_output_and_text_encoder_loop(gpu, pool_all):
     assert q.shape == (3, cfg.hidden_size) and c.shape == (2, cfg.hidden_size)
     again = enc.encode_queries(["x"], batch_size=1)
     assert abs(again[0] - q[2]).max() < 2e-2          # same text alone or inside a batch
+
+
+def test_model_loaded_from_reference_style_checkpoint_runs_identically(gpu, tmp_path):
+    """A Composer-style checkpoint file (state/model nesting, `model.bert.` prefixes, head keys) loaded through
+    the checkpoint loader gives bit-identical outputs to loading the plain state dict."""
+    import os
+    import m2_amd
+    cfg = m2_amd.m2_bert_80m(128)
+    cfg.num_hidden_layers = 1
+    sd = m2_amd.seeded_state_dict(cfg, 31)
+    path = os.path.join(tmp_path, "ckpt.pt")
+    wrapped = {"model.bert." + k: v for k, v in sd.items()}
+    wrapped["model.cls.predictions.bias"] = torch.zeros(8)
+    torch.save({"state": {"model": wrapped}}, path)
+    a = m2_amd.BertModel(cfg)
+    a.load_state_dict(sd)
+    b = m2_amd.BertModel(cfg)
+    missing, unexpected = m2_amd.load_reference_checkpoint(b, path)
+    assert missing == [] and unexpected == ["model.cls.predictions.bias"]
+    a, b = a.to(gpu).eval(), b.to(gpu).eval()
+    ids = torch.randint(0, cfg.vocab_size, (2, 128), generator=torch.Generator().manual_seed(4)).to(gpu)
+    (sa, pa), (sb, pb) = a(ids), b(ids)
+    assert torch.equal(sa, sb) and torch.equal(pa, pb)
