@@ -23,8 +23,10 @@
 // registers, twiddle, store in place".  The last forward pass and the first inverse pass are
 // radix-8 on contiguous groups of 8; thread w takes group g(w) AND the group g' that holds the
 // mirrored frequencies N-k, so the spectral multiply needs no exchange: it happens in registers
-// between the two radix-8 transforms.  The first forward pass reads straight from global memory
-// and the last inverse pass writes straight to global memory.
+// between the two radix-8 transforms.  Global memory is read and written 8 consecutive time steps per
+// thread (16-byte accesses); the row is staged in LDS between that layout and the first-pass layout.
+// This file serves sequence lengths up to 2048; longer rows use fftconv_split_kernels.hip (4096, 8192)
+// and fftconv_big_kernels.hip (32768).
 //
 // The filter spectra are stored in exactly the order the multiply consumes them
 // ("native order": spec[channel][slot 0..7][w 0..T-1] as float4 = K1.re, K1.im, K2.re, K2.im for the
@@ -322,14 +324,13 @@ static int launch_filter_spectrum(const float* taps1, const float* taps2, const 
   return check_launch("filter_spectrum");
 }
 
+// whole-row plans, N = 2L = 256 .. 4096 (longer rows go to the split half-transform kernels)
 #define M2_FOR_EACH_PLAN(X) \
   X(8, 4, 8, 1)             \
   X(9, 8, 8, 1)             \
   X(10, 16, 8, 1)           \
   X(11, 16, 16, 1)          \
-  X(12, 8, 8, 8)            \
-  X(13, 16, 8, 8)           \
-  X(14, 16, 16, 8)
+  X(12, 8, 8, 8)
 
 // N = 65536 (four sub-transforms per row), defined in fftconv_big_kernels.hip
 int launch_mixer_core_big_dispatch(const void* xproj, const float* u, const float* sw, const float* sb,
