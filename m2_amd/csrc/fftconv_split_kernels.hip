@@ -33,6 +33,17 @@
 
 namespace m2 {
 
+// LDS padding of the row buffer: two slots after every 32 and one more after every 512.  With it the staging
+// layout (32 consecutive slots per thread), the first pass (consecutive threads, consecutive slots at stride
+// L / R1) and the second pass (16 consecutive slots per 256) are all free of bank conflicts for 8-byte
+// accesses (checked by enumerating the 64 banks for every access pattern of the L = 8192 plan).
+__device__ __forceinline__ int sphys(int pos) { return pos + 2 * (pos >> 5) + (pos >> 9); }
+// Padded offset of logical offset `o` relative to a base position: valid where adding `o` to the base carries
+// neither into bit 5 nor into bit 9 from below (every access in this file: offsets are multiples of 256 on a
+// base below 256, multiples of 16 below 256 on a base whose low byte is below 16, or below 16 / 32 on a base
+// that is a multiple of 16 / 32).
+constexpr int spoff(int o) { return o + 2 * (o >> 5) + (o >> 9); }
+
 template <int LOGL_, int R1_, int R2_>
 struct SplitPlan {
   static constexpr int LOGL = LOGL_, L = 1 << LOGL_, N = 2 * L;
@@ -42,7 +53,7 @@ struct SplitPlan {
   static constexpr int M = L / RP;                // groups of 16 in the last pass
   static constexpr int S1 = L / R1, S2 = S1 / R2;
   static constexpr int NB1 = E / R1, NB2 = E / R2;
-  static constexpr int ROW_LDS = L + (L >> 4);    // padded complex slots of the row buffer
+  static constexpr int ROW_LDS = L + 2 * (L >> 5) + (L >> 9);    // padded complex slots of the row buffer
   static constexpr int TAB2 = R2 * S2;            // pass-2 twiddle table
   static constexpr int WG_LDS = ROW_LDS + TAB2;   // float2 slots per workgroup
   static_assert(R1 * R2 * RP == L, "radices must multiply to L");
@@ -133,10 +144,10 @@ template <class P>
 __device__ __forceinline__ void pass1_load(cf (&x)[32], int t, const float2* row) {
   static_for<0, P::NB1>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
-    const float2* pb = row + phys(t + P::T * i);
+    const float2* pb = row + sphys(t + P::T * i);
     static_for<0, P::R1>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
-      x[i * P::R1 + j] = lds_get(pb, poff(j * P::S1));
+      x[i * P::R1 + j] = lds_get(pb, spoff(j * P::S1));
     });
   });
 }
@@ -144,10 +155,10 @@ template <class P>
 __device__ __forceinline__ void pass1_store(const cf (&x)[32], int t, float2* row) {
   static_for<0, P::NB1>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
-    float2* pb = row + phys(t + P::T * i);
+    float2* pb = row + sphys(t + P::T * i);
     static_for<0, P::R1>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
-      lds_put(pb, poff(j * P::S1), x[i * P::R1 + j]);
+      lds_put(pb, spoff(j * P::S1), x[i * P::R1 + j]);
     });
   });
 }
@@ -166,12 +177,12 @@ __device__ __forceinline__ void fwd_pass1(cf (&x)[32], int t, float2* row, const
     dif<R, i * R, 32>(x);
     Pass1Powers<R> pw;
     pass1_powers<R, ODD>(b[i], pw);
-    float2* pb = row + phys(t + P::T * i);
+    float2* pb = row + sphys(t + P::T * i);
     static_for<0, R>([&](auto kk) {
       constexpr int k = decltype(kk)::value;
       cf v = x[i * R + bitrev(k, bits)];
       if constexpr (ODD || k > 0) v = cmul(v, pass1_twiddle<R, ODD, k>(pw));
-      lds_put(pb, poff(k * P::S1), v);
+      lds_put(pb, spoff(k * P::S1), v);
     });
   });
 }
@@ -184,10 +195,10 @@ __device__ __forceinline__ void inv_pass1(cf (&x)[32], int t, const float2* row,
     constexpr int i = decltype(ii)::value;
     Pass1Powers<R> pw;
     pass1_powers<R, ODD>(b[i], pw);
-    const float2* pb = row + phys(t + P::T * i);
+    const float2* pb = row + sphys(t + P::T * i);
     static_for<0, R>([&](auto kk) {
       constexpr int k = decltype(kk)::value;
-      cf v = lds_get(pb, poff(k * P::S1));
+      cf v = lds_get(pb, spoff(k * P::S1));
       if constexpr (ODD || k > 0) v = cmulc(v, pass1_twiddle<R, ODD, k>(pw));
       x[i * R + bitrev(k, bits)] = v;
     });
@@ -207,10 +218,10 @@ __device__ __forceinline__ void fwd_pass2(cf (&x)[32], int t, float2* row, const
   static_for<0, P::NB2>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
     const int q = t + P::T * i, blk = q / S, m = q % S;
-    float2* pb = row + phys(blk * (S * R) + m);
+    float2* pb = row + sphys(blk * (S * R) + m);
     static_for<0, R>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
-      x[i * R + j] = lds_get(pb, poff(j * S));
+      x[i * R + j] = lds_get(pb, spoff(j * S));
     });
     dif<R, i * R, 32>(x);
     static_for<0, R>([&](auto kk) {
@@ -220,7 +231,7 @@ __device__ __forceinline__ void fwd_pass2(cf (&x)[32], int t, float2* row, const
         const float2 w = tab2[k * S + m];
         v = cmul(v, cf{w.x, w.y});
       }
-      lds_put(pb, poff(k * S), v);
+      lds_put(pb, spoff(k * S), v);
     });
   });
 }
@@ -230,10 +241,10 @@ __device__ __forceinline__ void inv_pass2(cf (&x)[32], int t, float2* row, const
   static_for<0, P::NB2>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
     const int q = t + P::T * i, blk = q / S, m = q % S;
-    float2* pb = row + phys(blk * (S * R) + m);
+    float2* pb = row + sphys(blk * (S * R) + m);
     static_for<0, R>([&](auto kk) {
       constexpr int k = decltype(kk)::value;
-      cf v = lds_get(pb, poff(k * S));
+      cf v = lds_get(pb, spoff(k * S));
       if constexpr (k > 0) {
         const float2 w = tab2[k * S + m];
         v = cmulc(v, cf{w.x, w.y});
@@ -243,7 +254,7 @@ __device__ __forceinline__ void inv_pass2(cf (&x)[32], int t, float2* row, const
     dit<R, i * R, 32>(x);
     static_for<0, R>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
-      lds_put(pb, poff(j * S), x[i * R + j]);
+      lds_put(pb, spoff(j * S), x[i * R + j]);
     });
   });
 }
@@ -251,8 +262,8 @@ __device__ __forceinline__ void inv_pass2(cf (&x)[32], int t, float2* row, const
 // last pass: two contiguous groups of 16 per thread, radix 16 in registers (bit-reversed order)
 template <class P>
 __device__ __forceinline__ void fwd_groups(cf (&x)[32], const float2* row, int ga, int gb) {
-  const float2* pa = row + phys(ga * 16);
-  const float2* pb = row + phys(gb * 16);
+  const float2* pa = row + sphys(ga * 16);
+  const float2* pb = row + sphys(gb * 16);
   static_for<0, 16>([&](auto jj) {
     constexpr int j = decltype(jj)::value;
     x[j] = lds_get(pa, j);
@@ -265,8 +276,8 @@ template <class P>
 __device__ __forceinline__ void inv_groups(cf (&x)[32], float2* row, int ga, int gb) {
   dit<16, 0, 32>(x);
   dit<16, 16, 32>(x);
-  float2* pa = row + phys(ga * 16);
-  float2* pb = row + phys(gb * 16);
+  float2* pa = row + sphys(ga * 16);
+  float2* pb = row + sphys(gb * 16);
   static_for<0, 16>([&](auto jj) {
     constexpr int j = decltype(jj)::value;
     lds_put(pa, j, x[j]);
@@ -274,26 +285,47 @@ __device__ __forceinline__ void inv_groups(cf (&x)[32], float2* row, int ga, int
   });
 }
 
-// Work item w takes group g (second digit in its lower half) and, in the even half, the group with the
-// mirrored frequencies (L - k) mod L; in the odd half the complement group (frequencies L - 1 - k).
-// Work item 0 of the even half takes the two self-mirrored groups 0 and R2 / 2.
+// Groups of 16 taken by work item w in the last pass.  Group index g = k1 R2 + k2 holds the frequencies
+// k = k1 + R1 k2 + R1 R2 j (slot j).
+// Even half: the partner is the group with the mirrored frequencies (L - k) mod L.  Work items are dealt so that
+// consecutive items take consecutive groups (no LDS bank conflicts): first the groups with 1 <= k1 < R1/2 (all
+// k2), whose partners have k1 > R1/2; then k1 = 0 (partners inside k1 = 0: k2 <-> R2 - k2), where the item with
+// k2 = 0 is the special one that takes the two self-mirrored groups 0 and R2/2; then k1 = R1/2 (k2 <-> R2-1-k2).
+// Odd half: the partner is the complement group (frequencies L - 1 - k): item w takes group w and M - 1 - w.
 template <class P>
-__device__ __forceinline__ void split_groups(int w, int& g, int& g_mirror, int& g_comp) {
+struct SplitGroups {
+  int ge, gm;       // even half: group and mirrored group
+  int go, gc;       // odd half: group and complement group
+  bool special;     // even half: this item holds groups 0 and R2/2 (DC, Nyquist, self-mirrored slots)
+};
+template <class P>
+__device__ __forceinline__ SplitGroups<P> split_groups(int w) {
   constexpr int R1 = P::R1, R2 = P::R2;
-  g = (w / (R2 / 2)) * R2 + (w % (R2 / 2));
-  g_comp = P::M - 1 - g;
-  if (w == 0) {
-    g_mirror = R2 / 2;
-    return;
-  }
-  int k1 = g / R2, k2 = g % R2;
-  if (k1) {
-    k1 = R1 - k1;
-    k2 = R2 - 1 - k2;
+  constexpr int BULK = (R1 / 2 - 1) * R2;
+  SplitGroups<P> s;
+  s.go = w;
+  s.gc = P::M - 1 - w;
+  s.special = (w == BULK);
+  int k1, k2;
+  if (w < BULK) {
+    k1 = 1 + w / R2;
+    k2 = w % R2;
+  } else if (w < BULK + R2 / 2) {
+    k1 = 0;
+    k2 = w - BULK;
   } else {
-    k2 = R2 - k2;
+    k1 = R1 / 2;
+    k2 = w - BULK - R2 / 2;
   }
-  g_mirror = k1 * R2 + k2;
+  s.ge = k1 * R2 + k2;
+  if (s.special) {
+    s.gm = R2 / 2;
+  } else if (k1) {
+    s.gm = (R1 - k1) * R2 + (R2 - 1 - k2);
+  } else {
+    s.gm = R2 - k2;
+  }
+  return s;
 }
 
 // One spectral pair: za sits at frequency kappa, zb at N - kappa.  Returns W[kappa] in za and W[N - kappa] in
@@ -354,7 +386,8 @@ __device__ __forceinline__ void tab2_init(float2* tab2) {
 // in the first-pass layout at entry and exit, so halves can follow each other without a barrier.
 template <class P, bool ODD>
 __device__ __forceinline__ void half_convolution(cf (&x)[32], int t, float2* row, const float2* tab2,
-                                                 const cf (&b)[P::NB1], const float4* __restrict__ sp, int ga, int gb) {
+                                                 const cf (&b)[P::NB1], const float4* __restrict__ sp, int ga, int gb,
+                                                 bool special) {
   fwd_pass1<P, ODD>(x, t, row, b);
   phase_barrier();
   fwd_pass2<P>(x, t, row, tab2);
@@ -363,7 +396,7 @@ __device__ __forceinline__ void half_convolution(cf (&x)[32], int t, float2* row
   load_spectrum_batch<0>(K0, sp, P::T);
   fwd_groups<P>(x, row, ga, gb);
   __builtin_amdgcn_sched_barrier(0);
-  if (!ODD && t == 0) {
+  if (!ODD && special) {
     multiply_batch<true, 0>(x, K0);
     load_spectrum_batch<1>(K1, sp, P::T);
     multiply_batch<true, 1>(x, K1);
@@ -405,8 +438,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
   tab2_init<P>(tab2);
   cf b[P::NB1];
   static_for<0, P::NB1>([&](auto ii) { b[decltype(ii)::value] = unit_root(t + T * decltype(ii)::value, P::N); });
-  int g, gm, gc;
-  split_groups<P>(t, g, gm, gc);
+  const SplitGroups<P> grp = split_groups<P>(t);
   phase_barrier();
 
   // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each).  XCD e takes the channels
@@ -486,7 +518,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
         }
         gate.template set<q>(gt);
         const f32x4_t u0 = ru[2 * q], u1 = ru[2 * q + 1];
-        float2* dst = row + phys(n);       // 8 consecutive slots never straddle a pad
+        float2* dst = row + sphys(n);       // 8 consecutive slots never straddle a pad
         dst[0] = make_float2(a[0], u0.x); dst[1] = make_float2(a[1], u0.y);
         dst[2] = make_float2(a[2], u0.z); dst[3] = make_float2(a[3], u0.w);
         dst[4] = make_float2(a[4], u1.x); dst[5] = make_float2(a[5], u1.y);
@@ -501,14 +533,14 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
     static_for<0, 32>([&](auto ii) { held[decltype(ii)::value] = x[decltype(ii)::value]; });     // z, for the odd half
 
     const float4* sp = spec + (long)c * 32 * T + t;
-    half_convolution<P, false>(x, t, row, tab2, b, sp, g, gm);
+    half_convolution<P, false>(x, t, row, tab2, b, sp, grp.ge, grp.gm, grp.special);
     static_for<0, 32>([&](auto ii) {       // x <- z for the odd half, held <- the even half's result
       constexpr int i = decltype(ii)::value;
       const cf e = x[i];
       x[i] = held[i];
       held[i] = e;
     });
-    half_convolution<P, true>(x, t, row, tab2, b, sp + 16 * T, g, gc);
+    half_convolution<P, true>(x, t, row, tab2, b, sp + 16 * T, grp.go, grp.gc, false);
     static_for<0, 32>([&](auto ii) {
       constexpr int i = decltype(ii)::value;
       x[i] = cadd(x[i], held[i]);
@@ -520,7 +552,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
     static_for<0, 4>([&](auto qq) {
       constexpr int q = decltype(qq)::value;
       const int n = n0 + 8 * q;
-      const float2* src = row + phys(n);
+      const float2* src = row + sphys(n);
       float out[8];
       static_for<0, 8>([&](auto ee) {
         constexpr int e = decltype(ee)::value;
@@ -553,8 +585,7 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_split_kernel(
   tab2_init<P>(tab2);
   cf b[P::NB1];
   static_for<0, P::NB1>([&](auto ii) { b[decltype(ii)::value] = unit_root(t + T * decltype(ii)::value, P::N); });
-  int g, gm, gc;
-  split_groups<P>(t, g, gm, gc);
+  const SplitGroups<P> grp = split_groups<P>(t);
   // 1/N of the convolution, 1/2 of the separation of the two packed filters, 1/2 of the separation of the two
   // packed signals in the mixer kernel (pair_multiply_half)
   const float scale = 0.25f / (float)N;
@@ -596,7 +627,7 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_split_kernel(
         constexpr float sgn = ODD ? -1.f : 1.f;
         static_for<0, 8>([&](auto qq) {
           constexpr int q = decltype(qq)::value;
-          float2* dst = row + phys(4 * (q * T + t));     // 4 consecutive slots never straddle a pad
+          float2* dst = row + sphys(4 * (q * T + t));     // 4 consecutive slots never straddle a pad
           dst[0] = make_float2(lo1[q].x + sgn * hi1[q].x, lo2[q].x + sgn * hi2[q].x);
           dst[1] = make_float2(lo1[q].y + sgn * hi1[q].y, lo2[q].y + sgn * hi2[q].y);
           dst[2] = make_float2(lo1[q].z + sgn * hi1[q].z, lo2[q].z + sgn * hi2[q].z);
@@ -610,11 +641,11 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_split_kernel(
       __syncthreads();
       fwd_pass2<P>(x, t, row, tab2);
       __syncthreads();
-      fwd_groups<P>(x, row, g, ODD ? gc : gm);
+      fwd_groups<P>(x, row, ODD ? grp.go : grp.ge, ODD ? grp.gc : grp.gm);
       __syncthreads();      // LDS is restaged by the next half / channel
 
       float4* sp = spec + ((long)c * 2 + (ODD ? 1 : 0)) * 16 * T + t;
-      if (!ODD && t == 0) {
+      if (!ODD && grp.special) {
         const cf z0 = x[bitrev(0, 4)], zn = x[bitrev(8, 4)];
         sp[0] = make_float4(4.f * scale * z0.re, 4.f * scale * zn.re, 4.f * scale * z0.im, 4.f * scale * zn.im);
         static_for<1, 8>([&](auto ss) {
