@@ -141,6 +141,18 @@ int m2_blockdiag_linear_fwd(const void* x, const void* w, const float* bias, con
 int m2_layernorm_fwd(const float* x, const float* gamma, const float* beta, float eps, float* out_f32, void* out_bf16,
                      float* out_channel_major, int M, int d, void* stream);
 
+/* out = LayerNorm(blockdiag_multiply(x, w) + bias + residual) in one kernel: m2_blockdiag_linear_fwd followed by
+ * m2_layernorm_fwd without the fp32 intermediate (bert/src/bert_layers.py:504-506: wo, dropout, residual,
+ * layernorm).  Arguments as in those two; any of the three outputs may be NULL.
+ * m2_blockdiag_linear_layernorm_supported returns 1 for the shapes the fused kernel covers: nblocks == 4,
+ * (in_features / 4) % 64 == 0, (out_features / 4) % 32 == 0, out_features <= 768; for other shapes the fused
+ * entry point returns M2_ERR_UNSUPPORTED and the caller uses the two separate entry points. */
+int m2_blockdiag_linear_layernorm_supported(int in_features, int out_features, int nblocks);
+int m2_blockdiag_linear_layernorm_fwd(const void* x, const void* w, const float* bias, const void* residual,
+                                      const float* gamma, const float* beta, float eps, float* out_f32,
+                                      void* out_bf16, float* out_channel_major, int M, int in_features,
+                                      int out_features, int nblocks, void* stream);
+
 /* Embedding sum + LayerNorm in one pass (BertEmbeddings.forward in eval mode, bert/src/bert_layers.py:191-252):
  * row m = b L + l:  e = word_emb[input_ids[m]] + type_emb[token_type_ids[m]] (+ pos_emb[position_ids[m]]),
  * out = LayerNorm(e) in the same three forms as m2_layernorm_fwd (any may be NULL).

@@ -126,14 +126,26 @@ class BertGatedLinearUnitMLP(nn.Module):
     def ln_params(self):
         return self.layernorm.weight.detach().float(), self.layernorm.bias.detach().float(), self.layernorm.eps
 
+    def normed(self, a16: torch.Tensor, want_f32: bool, want_bf16: bool, want_channel_major: bool):
+        """a16 (M, d) bf16 -> LayerNorm(wo(glu(a16)) + bias + a16) in the requested forms (f32 | None, bf16 | None,
+        channel-major f32 | None).  `wo` and the LayerNorm are one kernel where the shape allows it."""
+        gamma, beta, eps = self.ln_params()
+        w = self.wo.weight_bf16()
+        nb, q, p = w.shape
+        if ops.blockdiag_linear_layernorm_supported(nb * p, nb * q, nb):
+            g = ops.blockdiag_glu(a16, self.gated_layers.weight_bf16())
+            return ops.blockdiag_linear_layernorm(g, w, self.wo.bias.detach().float().contiguous(), a16, gamma, beta, eps,
+                                                  want_f32=want_f32, want_bf16=want_bf16,
+                                                  want_channel_major=want_channel_major)
+        return ops.layernorm(self.presum(a16), gamma, beta, eps, want_f32=want_f32, want_bf16=want_bf16,
+                             want_channel_major=want_channel_major)
+
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
         if self.training and self.dropout.p > 0:
             raise NotImplementedError("m2_amd is a forward/inference path: call .eval() first")
         shape = hidden_states.shape
         a16 = hidden_states.reshape(-1, shape[-1]).to(torch.bfloat16).contiguous()
-        s = self.presum(a16)
-        gamma, beta, eps = self.ln_params()
-        o32, _, _ = ops.layernorm(s, gamma, beta, eps)
+        o32, _, _ = self.normed(a16, True, False, False)
         return o32.view(shape)
 
 
@@ -178,10 +190,8 @@ class BertLayer(nn.Module):
         if after_core is not None:
             after_core()
         a16 = torch.addmm(b_out, y.view(d, B * L).t(), w_out.t())                    # (M, d)
-        s = self.mlp.presum(a16)
-        gamma, beta, eps = self.mlp.ln_params()
         pre = at.hyena_training_additions        # the next layer then reads the fp32 form only
-        return ops.layernorm(s, gamma, beta, eps, want_f32=want_f32, want_bf16=not pre, want_channel_major=not pre)
+        return self.mlp.normed(a16, want_f32, not pre, not pre)
 
 
 class BertEncoder(nn.Module):

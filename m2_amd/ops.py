@@ -228,3 +228,32 @@ def embed_layernorm(input_ids: Tensor, token_type_ids: Optional[Tensor], positio
                                      _ptr(type_emb), _ptr(pos_emb), _ptr(gamma), _ptr(beta), float(eps), _ptr(o32),
                                      _ptr(o16), _ptr(ot), B, L, d, _stream()))
     return o32, o16, ot
+
+
+def blockdiag_linear_layernorm_supported(in_features: int, out_features: int, nblocks: int) -> bool:
+    return bool(lib.m2_blockdiag_linear_layernorm_supported(int(in_features), int(out_features), int(nblocks)))
+
+
+def blockdiag_linear_layernorm(x: Tensor, w: Tensor, bias: Optional[Tensor], residual: Optional[Tensor], gamma: Tensor,
+                               beta: Tensor, eps: float, want_f32: bool = True, want_bf16: bool = False,
+                               want_channel_major: bool = False):
+    """LayerNorm(blockdiag_multiply(x, w) + bias + residual) in one kernel, outputs as `layernorm`."""
+    M, in_f = x.shape
+    nb, q, p = w.shape
+    _require(x, "x", torch.bfloat16)
+    _require(w, "w", torch.bfloat16)
+    if nb * p != in_f:
+        raise ValueError(f"x has {in_f} features, weight expects {nb}*{p}")
+    d = nb * q
+    if bias is not None:
+        _require(bias, "bias", torch.float32, (d,))
+    if residual is not None:
+        _require(residual, "residual", torch.bfloat16, (M, d))
+    _require(gamma, "gamma", torch.float32, (d,))
+    _require(beta, "beta", torch.float32, (d,))
+    o32 = torch.empty(M, d, dtype=torch.float32, device=x.device) if want_f32 else None
+    o16 = torch.empty(M, d, dtype=torch.bfloat16, device=x.device) if want_bf16 else None
+    ot = torch.empty(d, M, dtype=torch.float32, device=x.device) if want_channel_major else None
+    check(lib.m2_blockdiag_linear_layernorm_fwd(_ptr(x), _ptr(w), _ptr(bias), _ptr(residual), _ptr(gamma), _ptr(beta),
+                                                float(eps), _ptr(o32), _ptr(o16), _ptr(ot), M, in_f, d, nb, _stream()))
+    return o32, o16, ot

@@ -396,3 +396,41 @@ def test_model_loaded_from_reference_style_checkpoint_runs_identically(gpu, tmp_
     ids = torch.randint(0, cfg.vocab_size, (2, 128), generator=torch.Generator().manual_seed(4)).to(gpu)
     (sa, pa), (sb, pb) = a(ids), b(ids)
     assert torch.equal(sa, sb) and torch.equal(pa, pb)
+
+
+@pytest.mark.parametrize("M,d,I", [(256, 768, 3072), (1000, 768, 3072), (64, 256, 1024), (130, 512, 768)])
+def test_blockdiag_linear_layernorm_fused(gpu, M, d, I):
+    """wo + bias + residual + LayerNorm as one kernel against fp64 on the bf16-rounded operands, all three output
+    forms, ragged M, and against the two separate kernels."""
+    from m2_amd import ops
+    nb = 4
+    assert ops.blockdiag_linear_layernorm_supported(I, d, nb)
+    assert not ops.blockdiag_linear_layernorm_supported(6144, 1536, nb)        # d > 768: separate kernels
+    assert not ops.blockdiag_linear_layernorm_supported(3072, 768, 8)
+    g = torch.Generator().manual_seed(M + d)
+    x = torch.randn(M, I, generator=g).bfloat16()
+    w = (torch.randn(nb, d // nb, I // nb, generator=g) * 0.05).bfloat16()
+    bias = torch.randn(d, generator=g)
+    resid = torch.randn(M, d, generator=g).bfloat16()
+    gamma = 1 + 0.1 * torch.randn(d, generator=g)
+    beta = 0.1 * torch.randn(d, generator=g)
+    xs = x.double().reshape(M, nb, I // nb)
+    s = torch.einsum("mkp,kqp->mkq", xs, w.double()).reshape(M, d) + bias.double() + resid.double()
+    want = torch.nn.functional.layer_norm(s, (d,), gamma.double(), beta.double(), 1e-12)
+    o32, o16, ot = ops.blockdiag_linear_layernorm(x.to(gpu), w.to(gpu), bias.to(gpu), resid.to(gpu), gamma.to(gpu),
+                                                  beta.to(gpu), 1e-12, want_f32=True, want_bf16=True, want_channel_major=True)
+    e, e2 = rel_err(o32, want)
+    assert e < 1e-3 and e2 < 1e-3, (e, e2)
+    assert torch.equal(ot, o32.t())
+    assert torch.equal(o16, o32.to(torch.bfloat16))
+    # the two separate kernels
+    s2 = ops.blockdiag_linear(x.to(gpu), w.to(gpu), bias.to(gpu), resid.to(gpu), out_dtype=torch.float32)
+    ref32, _, _ = ops.layernorm(s2, gamma.to(gpu), beta.to(gpu), 1e-12)
+    assert (ref32 - o32).abs().max().item() < 1e-4
+    # no bias, no residual, only the channel-major output
+    _, _, ot2 = ops.blockdiag_linear_layernorm(x.to(gpu), w.to(gpu), None, None, gamma.to(gpu), beta.to(gpu), 1e-5,
+                                               want_f32=False, want_bf16=False, want_channel_major=True)
+    s3 = torch.einsum("mkp,kqp->mkq", xs, w.double()).reshape(M, d)
+    want3 = torch.nn.functional.layer_norm(s3, (d,), gamma.double(), beta.double(), 1e-5)
+    e, e2 = rel_err(ot2.t(), want3)
+    assert e < 1e-3 and e2 < 1e-3, (e, e2)
