@@ -434,3 +434,101 @@ def test_blockdiag_linear_layernorm_fused(gpu, M, d, I):
     want3 = torch.nn.functional.layer_norm(s3, (d,), gamma.double(), beta.double(), 1e-5)
     e, e2 = rel_err(ot2.t(), want3)
     assert e < 1e-3 and e2 < 1e-3, (e, e2)
+
+
+@pytest.mark.parametrize("L", [128, 4096])
+@pytest.mark.parametrize("bidirectional,residual", [(False, True), (True, False), (False, False)])
+def test_mixer_variants_without_reverse_filter_or_residual_conv(gpu, L, bidirectional, residual):
+    """The module with bidirectional=False (reverse half of the window is zero) and / or residual_long_conv=False
+    (no second convolution, no u input), B = 1, on the whole-row (L = 128) and the split (L = 4096) kernels."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    d = 64
+    cfg = m2_amd.m2_bert_80m(L)
+    cfg.hidden_size, cfg.bidirectional, cfg.residual_long_conv = d, bidirectional, residual
+    sd = m2_amd.seeded_state_dict(cfg, 500 + L, std=0.1, what="mixer")
+    sd["in_linear.bias"] = torch.randn(3 * d, generator=torch.Generator().manual_seed(1)) * 0.1
+    mix = m2_amd.MonarchMixerSequenceMixing(d, l_max=L, bidirectional=bidirectional, hyena_emb_dim=5,
+                                            hyena_filter_order=128, residual_long_conv=residual, hyena_w=10, hyena_w_mod=1)
+    mix.load_state_dict(sd)
+    mix = mix.to(gpu).eval()
+    u = torch.randn(1, L, d, generator=torch.Generator().manual_seed(3))
+    y, _ = mix(u.to(gpu))
+    assert ("filter_fn2.bias" in sd) == residual
+    ref = O.mixer_forward(sd, "", u, bidirectional, residual)
+    e, e2 = rel_err(y, ref)
+    assert e < TOL_F32 and e2 < TOL_F32, (e, e2)
+
+
+def test_plain_fftconv_long_rows(gpu):
+    """m2_fftconv_fwd (one filter, no short conv, no gates) on the split kernels, fp32 and bf16 storage."""
+    from m2_amd import ops
+    from oracle import m2_oracle as O
+    for L in (4096, 8192):
+        d, B = 16, 2
+        g = torch.Generator().manual_seed(L)
+        x = torch.randn(d, B, L, generator=g)
+        t = torch.linspace(0, 1, 2 * L)
+        taps = torch.randn(d, 2 * L, generator=g) * torch.exp(-6 * torch.minimum(t, 1 - t))
+        D = torch.randn(d, generator=g)
+        spec = ops.filter_spectrum(taps.to(gpu), None, D.to(gpu), None)
+        ref = O.fftconv(x.double().permute(1, 0, 2), taps.double(), D.double()[None, :, None]).permute(1, 0, 2)
+        y = ops.fftconv(x.to(gpu), spec, B, L, d)
+        assert rel_err(y, ref)[0] < TOL_F32
+        y16 = ops.fftconv(x.bfloat16().to(gpu), spec, B, L, d)
+        ref16 = O.fftconv(x.bfloat16().double().permute(1, 0, 2), taps.double(), D.double()[None, :, None]).permute(1, 0, 2)
+        assert rel_err(y16.float(), ref16)[0] < 6e-3
+
+
+def test_mixer_core_full_size_impulse_and_linearity(gpu):
+    """At the benchmark's own size (L = 8192, B = 4, d = 768), properties that need no CPU transform:
+    (1) with the projections zeroed the core is the second bidirectional convolution alone, so a unit impulse at
+        position n0 must return the filter itself: y[t] = k_fwd[t - n0] for t >= n0, k_rev[n0 - t - 1] for t < n0
+        (+ D at t = n0);
+    (2) the core is affine in u: y(u1 + u2) - y(u1) - y(u2) + y(0) = 0."""
+    from m2_amd import ops
+    L, B, d = 8192, 4, 768
+    g = torch.Generator().manual_seed(77)
+    t = torch.linspace(0, 1, 2 * L)
+    taps = [(torch.randn(d, 2 * L, generator=g) * torch.exp(-5 * torch.minimum(t, 1 - t))).to(gpu) for _ in range(2)]
+    D = [torch.randn(d, generator=g).to(gpu) for _ in range(2)]
+    spec = ops.filter_spectrum(taps[0], taps[1], D[0], D[1])
+    sw = (torch.randn(3 * d, 3, generator=g) * 0.5).to(gpu)
+    sb = (torch.randn(3 * d, generator=g) * 0.1).to(gpu)
+    zero_x = torch.zeros(3 * d, B, L, device=gpu)
+    zero_b = torch.zeros(3 * d, device=gpu)
+    n0s = [0, 1, 4095, 8191]
+    u = torch.zeros(d, B, L, device=gpu)
+    for b, n0 in enumerate(n0s):
+        u[:, b, n0] = 1.0
+    y = ops.mixer_core(zero_x, u, sw, zero_b, spec, B, L, d)      # short conv of zeros with zero bias: a = 0, gate = 0
+    k = taps[1]
+    for b, n0 in enumerate(n0s):
+        want = torch.empty(d, L, device=gpu)
+        want[:, n0:] = k[:, :L - n0]                                 # causal taps k_fwd[t - n0]
+        if n0 > 0:
+            want[:, :n0] = k[:, 2 * L - n0:]                         # window position 2L - (n0 - t) holds k_rev[n0 - t - 1]
+        want[:, n0] += D[1]
+        err = (y[:, b] - want).abs().max().item() / want.abs().max().item()
+        assert err < TOL_F32, (n0, err)
+    # affinity in u with everything switched on
+    xproj = torch.randn(3 * d, B, L, generator=g).to(gpu)
+    u1 = torch.randn(d, B, L, generator=g).to(gpu)
+    u2 = torch.randn(d, B, L, generator=g).to(gpu)
+    f = lambda uu: ops.mixer_core(xproj, uu, sw, sb, spec, B, L, d)
+    resid = f(u1 + u2) - f(u1) - f(u2) + f(torch.zeros_like(u1))
+    scale = f(u1).abs().max().item()
+    assert resid.abs().max().item() / scale < 5e-5
+
+
+def test_unsupported_sizes_fail_loudly(gpu):
+    from m2_amd import ops
+    d = 64
+    taps = torch.zeros(d, 2 * 192, device=gpu)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.filter_spectrum(taps, None, None, None)                 # L = 192 is not a power of two
+    taps = torch.zeros(d, 2 * 16384, device=gpu)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.filter_spectrum(taps, None, None, None)                 # L = 16384 has no plan
+    with pytest.raises(RuntimeError):
+        ops.layernorm(torch.zeros(4, 100, device=gpu), torch.ones(100, device=gpu), torch.zeros(100, device=gpu), 1e-5)
