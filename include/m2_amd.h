@@ -79,8 +79,9 @@ int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int 
  * native counterpart in the reference: flashmm.mm_block_fwd (csrc/flashmm/flash_mm.cpp:70-226).
  * ------------------------------------------------------------------------------------------- */
 
-/* 1 if sequence length L is supported: 2L a power of two in [256, 16384] (one LDS-resident FFT per
- * row) or 2L = 65536 (four LDS-resident sub-transforms per row). */
+/* 1 if sequence length L is supported: a power of two in [128, 32768] (one LDS-resident transform per
+ * row up to 1024, two half-length transforms per row for 2048 .. 16384, four LDS-resident
+ * sub-transforms per row for 32768). */
 int m2_fftconv_supported_seqlen(int L);
 
 /* Bytes of the opaque spectrum buffer for d channels and sequence length L (both filters). */

@@ -25,7 +25,7 @@
 // mirrored frequencies N-k, so the spectral multiply needs no exchange: it happens in registers
 // between the two radix-8 transforms.  Global memory is read and written 8 consecutive time steps per
 // thread (16-byte accesses); the row is staged in LDS between that layout and the first-pass layout.
-// This file serves sequence lengths up to 2048; longer rows use fftconv_split_kernels.hip (4096, 8192)
+// This file serves sequence lengths up to 1024; longer rows use fftconv_split_kernels.hip (2048 .. 16384)
 // and fftconv_big_kernels.hip (32768).
 //
 // The filter spectra are stored in exactly the order the multiply consumes them
@@ -329,8 +329,7 @@ static int launch_filter_spectrum(const float* taps1, const float* taps2, const 
   X(8, 4, 8, 1)             \
   X(9, 8, 8, 1)             \
   X(10, 16, 8, 1)           \
-  X(11, 16, 16, 1)          \
-  X(12, 8, 8, 8)
+  X(11, 16, 16, 1)
 
 // N = 65536 (four sub-transforms per row), defined in fftconv_big_kernels.hip
 int launch_mixer_core_big_dispatch(const void* xproj, const float* u, const float* sw, const float* sb,
@@ -352,7 +351,7 @@ using namespace m2;
 
 extern "C" int m2_fftconv_supported_seqlen(int L) {
   int n = 2 * L;
-  return (n >= 256 && n <= 65536 && n != 32768 && (n & (n - 1)) == 0) ? 1 : 0;
+  return (n >= 256 && n <= 65536 && (n & (n - 1)) == 0) ? 1 : 0;
 }
 
 extern "C" size_t m2_filter_spectrum_bytes(int d, int L) {
@@ -364,7 +363,7 @@ extern "C" int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, co
   if (!taps1 || !spec) return set_error(M2_ERR_ARG, "m2_filter_spectrum_fwd: null pointer");
   if (d <= 0) return set_error(M2_ERR_ARG, "m2_filter_spectrum_fwd: d must be positive, got %d", d);
   if (!m2_fftconv_supported_seqlen(L))
-    return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: L=%d unsupported (need 2L a power of two in [256, 16384], or 65536)", L);
+    return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: L=%d unsupported (need L a power of two in [128, 32768])", L);
   const int logn = ilog2(2 * L);
   if (logn == 16) return launch_filter_spectrum_big(taps1, taps2, D1, D2, spec, d, (hipStream_t)stream);
   if (split_plan_exists(L)) return launch_filter_spectrum_split(taps1, taps2, D1, D2, spec, d, L, (hipStream_t)stream);
@@ -386,7 +385,7 @@ extern "C" int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, cons
   if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
     return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
   if (!m2_fftconv_supported_seqlen(L))
-    return set_error(M2_ERR_UNSUPPORTED, "m2_mixer_core_fwd: L=%d unsupported (need 2L a power of two in [256, 16384], or 65536)", L);
+    return set_error(M2_ERR_UNSUPPORTED, "m2_mixer_core_fwd: L=%d unsupported (need L a power of two in [128, 32768])", L);
   const int logn = ilog2(2 * L);
   hipStream_t s = (hipStream_t)stream;
   if (logn == 16) return launch_mixer_core_big_dispatch(xproj, u, short_w, short_b, proj_bias, spec, y, B, d, act_dtype, s);
@@ -410,7 +409,7 @@ extern "C" int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, 
   if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
     return set_error(M2_ERR_ARG, "m2_fftconv_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
   if (!m2_fftconv_supported_seqlen(L))
-    return set_error(M2_ERR_UNSUPPORTED, "m2_fftconv_fwd: L=%d unsupported (need 2L a power of two in [256, 16384], or 65536)", L);
+    return set_error(M2_ERR_UNSUPPORTED, "m2_fftconv_fwd: L=%d unsupported (need L a power of two in [128, 32768])", L);
   const int logn = ilog2(2 * L);
   hipStream_t s = (hipStream_t)stream;
   if (logn == 16) return launch_mixer_core_big_dispatch(x, nullptr, nullptr, nullptr, nullptr, spec, y, B, d, act_dtype, s);

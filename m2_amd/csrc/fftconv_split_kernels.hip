@@ -1,4 +1,4 @@
-// Long sequences (L = 4096, 8192, 16384): the fused mixer core and the filter-spectrum kernel with the
+// Long sequences (L = 2048 .. 16384): the fused mixer core and the filter-spectrum kernel with the
 // row's N = 2L point transform split by frequency parity into two L-point half transforms that run one
 // after the other through one L-point LDS buffer.
 //
@@ -685,7 +685,7 @@ static int launch_mixer_split(const void* xproj, const float* u, const float* sw
   const int rows_per_xcd = (d / 8) * B;
   int per_cu = (int)((160 * 1024) / lds_bytes);
   if (per_cu < 1) per_cu = 1;
-  if (per_cu > 4) per_cu = 4;
+  if (per_cu > 512 / P::T) per_cu = 512 / P::T;  // two waves per SIMD at 256 registers
   int slots = (num_cus() / 8) * per_cu;          // workgroups per XCD
   if (slots > rows_per_xcd) slots = rows_per_xcd;
   hipLaunchKernelGGL(kern, dim3(8 * slots), dim3(P::T), lds_bytes, stream, (const ACT*)xproj, u, sw, sb, pbias,
@@ -704,7 +704,7 @@ static int launch_filter_spectrum_split_t(const float* taps1, const float* taps2
   }
   int per_cu = (int)((160 * 1024) / lds_bytes);
   if (per_cu < 1) per_cu = 1;
-  if (per_cu > 4) per_cu = 4;
+  if (per_cu > 512 / P::T) per_cu = 512 / P::T;
   int grid = num_cus() * per_cu;
   if (grid > 2 * d) grid = 2 * d;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(P::T), lds_bytes, stream, taps1, taps2, D1, D2, (float4*)spec, d);
@@ -712,8 +712,10 @@ static int launch_filter_spectrum_split_t(const float* taps1, const float* taps2
 }
 
 #define M2_FOR_EACH_SPLIT_PLAN(X) \
+  X(11, 16, 8)                    \
   X(12, 16, 16)                   \
-  X(13, 32, 16)
+  X(13, 32, 16)                   \
+  X(14, 32, 32)
 
 bool split_plan_exists(int L) {
   switch (L) {

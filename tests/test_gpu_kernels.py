@@ -54,14 +54,14 @@ def test_hyena_filter_taps(gpu, L, std):
         assert rel_err(hr.cpu(), kr.T[None])[0] < max(2e-5, 4 * e32)
 
 
-@pytest.mark.parametrize("L", [128, 256, 512, 1024, 2048, 4096, 8192, 32768])
+@pytest.mark.parametrize("L", [128, 256, 512, 1024, 2048, 4096, 8192, 16384, 32768])
 @pytest.mark.parametrize("act", ["f32", "bf16"])
 def test_mixer_core(gpu, L, act):
     """K1c + K2 vs the oracle's short conv / gating / two fftconvs, every FFT plan."""
     import m2_amd
     from m2_amd import ops
     from oracle import m2_oracle as O
-    d, B = (64, 3) if L <= 8192 else (16, 2)
+    d, B = (64, 3) if L <= 16384 else (16, 2)
     g = torch.Generator().manual_seed(100 + L)
     dt = torch.float32 if act == "f32" else torch.bfloat16
     xproj = torch.randn(3 * d, B, L, generator=g).to(dt)
@@ -157,7 +157,7 @@ def test_config1_mixer_fp32(gpu):
     assert e < TOL_F32 and e2 < TOL_F32, (e, e2)
 
 
-@pytest.mark.parametrize("L,B,layers", [(128, 4, 2), (1024, 2, 2), (32768, 1, 1)])
+@pytest.mark.parametrize("L,B,layers", [(128, 4, 2), (1024, 2, 2), (16384, 1, 1), (32768, 1, 1)])
 def test_encoder_small(gpu, L, B, layers):
     """Fused encoder schedule and the module-by-module path agree with the oracle (bf16 tolerance)."""
     import m2_amd
@@ -527,8 +527,26 @@ def test_unsupported_sizes_fail_loudly(gpu):
     taps = torch.zeros(d, 2 * 192, device=gpu)
     with pytest.raises(RuntimeError, match="unsupported"):
         ops.filter_spectrum(taps, None, None, None)                 # L = 192 is not a power of two
-    taps = torch.zeros(d, 2 * 16384, device=gpu)
+    taps = torch.zeros(d, 2 * 64, device=gpu)
     with pytest.raises(RuntimeError, match="unsupported"):
-        ops.filter_spectrum(taps, None, None, None)                 # L = 16384 has no plan
+        ops.filter_spectrum(taps, None, None, None)                 # L = 64 is below the shortest plan
     with pytest.raises(RuntimeError):
         ops.layernorm(torch.zeros(4, 100, device=gpu), torch.ones(100, device=gpu), torch.zeros(100, device=gpu), 1e-5)
+
+
+@pytest.mark.parametrize("extra", [["--config", "c3"], ["--config", "c2", "--eager"]])
+def test_bench_prints_its_json_line(gpu, extra):
+    """bench.py as a child process (2 timed steps, no CPU leg): one JSON line with the fields the contract names."""
+    import json, os, subprocess, sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "2", "--warmup", "1",
+                        "--no-cpu-baseline"] + extra, capture_output=True, text=True, timeout=110, cwd=root)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = json.loads(r.stdout.strip().splitlines()[-1])
+    assert line["n_gpus"] == 1 and line["steps"] == 2 and line["value"] > 0 and line["unit"] == "seq/s"
+    roof = line["roofline"]
+    assert roof["bound"] == "hbm" and 0 < roof["frac"] < 1 and roof["peak"] == 8000.0
+    assert abs(roof["achieved"] / roof["peak"] - roof["frac"]) < 1e-9
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=60, cwd=root)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
