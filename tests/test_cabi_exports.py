@@ -36,7 +36,8 @@ def test_size_queries_and_argument_checks_without_gpu():
     assert lib.m2_fftconv_supported_seqlen(128) == 1
     assert lib.m2_fftconv_supported_seqlen(8192) == 1
     assert lib.m2_fftconv_supported_seqlen(32768) == 1
-    assert lib.m2_fftconv_supported_seqlen(16384) == 0
+    assert lib.m2_fftconv_supported_seqlen(16384) == 1
+    assert lib.m2_fftconv_supported_seqlen(64) == 0 and lib.m2_fftconv_supported_seqlen(65536) == 0
     assert lib.m2_fftconv_supported_seqlen(65536) == 0
     assert lib.m2_fftconv_supported_seqlen(64) == 0
     assert lib.m2_fftconv_supported_seqlen(100) == 0
