@@ -26,7 +26,7 @@
 // between the two radix-8 transforms.  Global memory is read and written 8 consecutive time steps per
 // thread (16-byte accesses); the row is staged in LDS between that layout and the first-pass layout.
 // This file serves sequence lengths up to 1024; longer rows use fftconv_split_kernels.hip (2048 .. 16384)
-// and fftconv_big_kernels.hip (32768).
+// and fftconv_real_kernels.hip (32768).
 //
 // The filter spectra are stored in exactly the order the multiply consumes them
 // ("native order": spec[channel][slot 0..7][w 0..T-1] as float4 = K1.re, K1.im, K2.re, K2.im for the
@@ -331,14 +331,14 @@ static int launch_filter_spectrum(const float* taps1, const float* taps2, const 
   X(10, 16, 8, 1)           \
   X(11, 16, 16, 1)
 
-// N = 65536 (four sub-transforms per row), defined in fftconv_big_kernels.hip
-int launch_mixer_core_big_dispatch(const void* xproj, const float* u, const float* sw, const float* sb,
-                                   const float* pbias, const float* spec, void* y, int B, int d, int act_dtype,
-                                   hipStream_t stream);
-int launch_filter_spectrum_big(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
-                               int d, hipStream_t stream);
+// L = 32768 (every real signal on its own, as half transforms of 16384 points), defined in fftconv_real_kernels.hip
+size_t real_spectrum_bytes(int d);
+int launch_mixer_real_dispatch(const void* xproj, const float* u, const float* sw, const float* sb, const float* pbias,
+                               const float* spec, void* y, int B, int d, int act_dtype, hipStream_t stream);
+int launch_filter_spectrum_real(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
+                                int d, hipStream_t stream);
 
-// L = 4096, 8192: even/odd split half transforms, defined in fftconv_split_kernels.hip
+// L = 2048 .. 16384: even/odd split half transforms, defined in fftconv_split_kernels.hip
 bool split_plan_exists(int L);
 int launch_mixer_split_dispatch(const void* xproj, const float* u, const float* sw, const float* sb, const float* pbias,
                                 const float* spec, void* y, int B, int L, int d, int act_dtype, hipStream_t stream);
@@ -355,6 +355,7 @@ extern "C" int m2_fftconv_supported_seqlen(int L) {
 }
 
 extern "C" size_t m2_filter_spectrum_bytes(int d, int L) {
+  if (L == 32768) return real_spectrum_bytes(d);      // (Ke, Ko, w Ko) per frequency pair and filter
   return (size_t)d * (size_t)L * 16;        // d channels x 8 slots x (2L/16) work items x float4
 }
 
@@ -365,7 +366,7 @@ extern "C" int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, co
   if (!m2_fftconv_supported_seqlen(L))
     return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: L=%d unsupported (need L a power of two in [128, 32768])", L);
   const int logn = ilog2(2 * L);
-  if (logn == 16) return launch_filter_spectrum_big(taps1, taps2, D1, D2, spec, d, (hipStream_t)stream);
+  if (logn == 16) return launch_filter_spectrum_real(taps1, taps2, D1, D2, spec, d, (hipStream_t)stream);
   if (split_plan_exists(L)) return launch_filter_spectrum_split(taps1, taps2, D1, D2, spec, d, L, (hipStream_t)stream);
   switch (logn) {
 #define X(LOGN, R1, R2, R3) \
@@ -388,7 +389,7 @@ extern "C" int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, cons
     return set_error(M2_ERR_UNSUPPORTED, "m2_mixer_core_fwd: L=%d unsupported (need L a power of two in [128, 32768])", L);
   const int logn = ilog2(2 * L);
   hipStream_t s = (hipStream_t)stream;
-  if (logn == 16) return launch_mixer_core_big_dispatch(xproj, u, short_w, short_b, proj_bias, spec, y, B, d, act_dtype, s);
+  if (logn == 16) return launch_mixer_real_dispatch(xproj, u, short_w, short_b, proj_bias, spec, y, B, d, act_dtype, s);
   if (split_plan_exists(L)) return launch_mixer_split_dispatch(xproj, u, short_w, short_b, proj_bias, spec, y, B, L, d, act_dtype, s);
   switch (logn) {
 #define X(LOGN, R1, R2, R3)                                                                                       \
@@ -412,7 +413,7 @@ extern "C" int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, 
     return set_error(M2_ERR_UNSUPPORTED, "m2_fftconv_fwd: L=%d unsupported (need L a power of two in [128, 32768])", L);
   const int logn = ilog2(2 * L);
   hipStream_t s = (hipStream_t)stream;
-  if (logn == 16) return launch_mixer_core_big_dispatch(x, nullptr, nullptr, nullptr, nullptr, spec, y, B, d, act_dtype, s);
+  if (logn == 16) return launch_mixer_real_dispatch(x, nullptr, nullptr, nullptr, nullptr, spec, y, B, d, act_dtype, s);
   if (split_plan_exists(L)) return launch_mixer_split_dispatch(x, nullptr, nullptr, nullptr, nullptr, spec, y, B, L, d, act_dtype, s);
   switch (logn) {
 #define X(LOGN, R1, R2, R3)                                                                                  \
