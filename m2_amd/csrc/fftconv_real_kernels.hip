@@ -55,12 +55,12 @@ __device__ __forceinline__ cf self_multiply_real(cf z, float ke, float ko, float
   return {z.re * ke + z.im * kw, z.re * ko + z.im * ke};
 }
 
-// spectral multiply of the 16 + 16 points a thread holds after fwd_groups, slots 8 HB .. 8 HB + 7 (same
+// spectral multiply of the 16 + 16 points a thread holds after fwd_groups, slots 4 HB .. 4 HB + 3 (same
 // pairing as multiply_batch in fft_split.h)
 template <bool EVEN_SPECIAL, int HB>
-__device__ __forceinline__ void multiply_batch_real(cf (&x)[32], const float4 (&K)[8], const float2 (&W)[8]) {
-  static_for<0, 8>([&](auto ss) {
-    constexpr int s = 8 * HB + decltype(ss)::value;
+__device__ __forceinline__ void multiply_batch_real(cf (&x)[32], const float4 (&K)[4], const float2 (&W)[4]) {
+  static_for<0, 4>([&](auto ss) {
+    constexpr int s = 4 * HB + decltype(ss)::value;
     const float4 k = K[decltype(ss)::value];
     const float2 w = W[decltype(ss)::value];
     if constexpr (!EVEN_SPECIAL) {
@@ -77,16 +77,17 @@ __device__ __forceinline__ void multiply_batch_real(cf (&x)[32], const float4 (&
   });
 }
 template <int HB>
-__device__ __forceinline__ void load_spectrum_batch_real(float4 (&K)[8], float2 (&W)[8], const float4* __restrict__ sp4,
+__device__ __forceinline__ void load_spectrum_batch_real(float4 (&K)[4], float2 (&W)[4], const float4* __restrict__ sp4,
                                                          const float2* __restrict__ sp2, int T) {
-  static_for<0, 8>([&](auto s) {
-    K[decltype(s)::value] = sp4[(8 * HB + decltype(s)::value) * T];
-    W[decltype(s)::value] = sp2[(8 * HB + decltype(s)::value) * T];
+  static_for<0, 4>([&](auto s) {
+    K[decltype(s)::value] = sp4[(4 * HB + decltype(s)::value) * T];
+    W[decltype(s)::value] = sp2[(4 * HB + decltype(s)::value) * T];
   });
 }
 
 // One half transform of one real signal: forward passes from registers (first-pass layout), polyphase multiply,
-// inverse passes back to registers.  Same barrier structure as half_convolution in fft_split.h.
+// inverse passes back to registers.  Same barrier structure as half_convolution in fft_split.h; the spectrum
+// comes in four batches, each loaded while the one before it is multiplied.
 template <class P, bool ODD>
 __device__ __forceinline__ void half_convolution_real(cf (&x)[32], int t, float2* row, const float2* tab2,
                                                       const cf (&b)[P::NB1], const float4* __restrict__ sp4,
@@ -95,20 +96,23 @@ __device__ __forceinline__ void half_convolution_real(cf (&x)[32], int t, float2
   phase_barrier();
   fwd_pass2<P>(x, t, row, tab2);
   phase_barrier();
-  float4 K0[8], K1[8];
-  float2 W0[8], W1[8];
-  load_spectrum_batch_real<0>(K0, W0, sp4, sp2, P::T);
+  float4 Ka[4], Kb[4];
+  float2 Wa[4], Wb[4];
+  load_spectrum_batch_real<0>(Ka, Wa, sp4, sp2, P::T);
   fwd_groups<P>(x, row, ga, gb);
   __builtin_amdgcn_sched_barrier(0);
-  if (!ODD && special) {
-    multiply_batch_real<true, 0>(x, K0, W0);
-    load_spectrum_batch_real<1>(K1, W1, sp4, sp2, P::T);
-    multiply_batch_real<true, 1>(x, K1, W1);
-  } else {
-    multiply_batch_real<false, 0>(x, K0, W0);
-    load_spectrum_batch_real<1>(K1, W1, sp4, sp2, P::T);
-    multiply_batch_real<false, 1>(x, K1, W1);
-  }
+  auto multiply = [&](auto sp) __attribute__((always_inline)) {
+    constexpr bool S = decltype(sp)::value == 1;
+    load_spectrum_batch_real<1>(Kb, Wb, sp4, sp2, P::T);
+    multiply_batch_real<S, 0>(x, Ka, Wa);
+    load_spectrum_batch_real<2>(Ka, Wa, sp4, sp2, P::T);
+    multiply_batch_real<S, 1>(x, Kb, Wb);
+    load_spectrum_batch_real<3>(Kb, Wb, sp4, sp2, P::T);
+    multiply_batch_real<S, 2>(x, Ka, Wa);
+    multiply_batch_real<S, 3>(x, Kb, Wb);
+  };
+  if (!ODD && special) multiply(ic<1>{});
+  else multiply(ic<0>{});
   __builtin_amdgcn_sched_barrier(0);
   inv_groups<P>(x, row, ga, gb);
   phase_barrier();
@@ -227,7 +231,8 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
   const int rows_per_xcd = (d >> 3) * B;
   for (int j = slot; j < rows_per_xcd; j += slots) {
-    const int c = (j / B) * 8 + xcd, bb = j % B;
+    // the same for every lane: say so, so that row base addresses live in scalar registers
+    const int c = __builtin_amdgcn_readfirstlane((j / B) * 8 + xcd), bb = __builtin_amdgcn_readfirstlane(j % B);
     const float* spc = spec + (long)c * 4 * BLK;
     cf x[32], acc[32];
 
@@ -272,6 +277,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
     });
 
     // ---- gate: acc = y1 * sc(x2)
+    __builtin_amdgcn_sched_barrier(0);
     if constexpr (FULL) {
       float w2[3];
 #pragma unroll
@@ -285,6 +291,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
     }
 
     // ---- second signal: the layer input u, convolved with filter 2; its two half transforms are added to acc
+    __builtin_amdgcn_sched_barrier(0);
     if constexpr (HAS_U) {
       const float* pu = uin + ((long)c * B + bb) * LS;
       load_slots<P, float>(pu, t, x);
@@ -297,7 +304,10 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
         constexpr int r = decltype(rr)::value;
         acc[r] = cadd(acc[r], x[r]);
       });
-      load_slots<P, float>(pu, t, x);
+      __builtin_amdgcn_sched_barrier(0);
+      int again = 0;
+      asm volatile("" : "+v"(again));    // a second load, not the first one's registers kept across the half transform
+      load_slots<P, float>(pu + again, t, x);
       {
         const float4* sp4 = reinterpret_cast<const float4*>(spc + 3 * BLK) + t;
         const float2* sp2 = reinterpret_cast<const float2*>(spc + 3 * BLK + 64L * T) + t;
