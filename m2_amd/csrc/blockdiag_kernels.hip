@@ -496,21 +496,175 @@ __global__ __launch_bounds__(256) void blockdiag_glu_ws_kernel(const uint16_t* _
   store_tile((s - 1) & 1, m_begin + 32 * (s - 1));
 }
 
+// The same kernel software-pipelined inside every wave: two accumulator sets, and the MFMAs of slab s + 1
+// sit in the same basic block as the gelu(gate) * value epilogue of slab s, so that the vector ALU works in the
+// shadow of the matrix pipe (the epilogue costs more vector-ALU cycles than the product costs MFMA cycles, and
+// with one accumulator set the two were measured to run one after the other).
+// NW waves per workgroup, 32 NW output columns: every column slice reads all of x again (from L2), so wider
+// workgroups cut that traffic.
+template <int KS, int NW>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void blockdiag_glu_ws3_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                                uint16_t* __restrict__ out, int M, int nb, int q,
+                                                                int rows_per_wg) {
+  constexpr int p = 16 * KS;
+  constexpr int AROW = p + 8;                       // padded bf16 row of an A slab
+  constexpr int NT = 64 * NW, NC = 32 * NW;         // threads, output columns
+  constexpr int GROW = NC + 8;                      // padded bf16 row of the result tile
+  constexpr int CPR = 2 * (p / 8);                  // 16-byte chunks per slab row (gate K-range then value K-range)
+  constexpr int NCH = 32 * CPR / NT;                // chunks per thread per slab
+  constexpr int ABUF = 2 * 32 * AROW;               // bf16 elements of one A buffer
+  static_assert((32 * CPR) % NT == 0, "slab must divide over the threads");
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  uint16_t* sA = smem;                              // [2][2][32][AROW]
+  // a separate object, so that the compiler may move the epilogue's writes past the product's operand reads
+  __shared__ __attribute__((aligned(16))) uint16_t sG[2 * 32 * GROW];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
+  const int I = nb * q / 2, in_f = nb * p;
+  const int nslices = I / NC;
+  int slice, chunk;
+  {
+    const int nchunks = (M + rows_per_wg - 1) / rows_per_wg;
+    const int id = blockIdx.x, e = id & 7, l = id >> 3;
+    const int full = (nchunks / 8) * 8;
+    if (id < full * nslices) { chunk = (l / nslices) * 8 + e; slice = l % nslices; }
+    else { const int rid = id - full * nslices; chunk = full + rid / nslices; slice = rid % nslices; }
+  }
+  const int n0 = slice * NC;
+  const int blk = n0 / q, jj = n0 % q;
+  const int m_begin = chunk * rows_per_wg;
+  const int m_end = min(M, m_begin + rows_per_wg);
+  const int nslab = (m_end - m_begin + 31) / 32;
+
+  bf16x8 bwg[KS], bwv[KS];
+  {
+    const uint16_t* wg = w + ((long)blk * q + jj + 32 * wave + i32) * p + 8 * half;
+    const uint16_t* wv = wg + (long)(nb / 2) * q * p;
+    static_for<0, KS>([&](auto kk) {
+      bwg[decltype(kk)::value] = ld8(wg + 16 * decltype(kk)::value);
+      bwv[decltype(kk)::value] = ld8(wv + 16 * decltype(kk)::value);
+    });
+  }
+  int crow[NCH], ccol[NCH], clds[NCH];
+  static_for<0, NCH>([&](auto jj_) {
+    constexpr int j = decltype(jj_)::value;
+    const int id = tid + NT * j, r = id / CPR, c = id % CPR, m2 = c / (p / 8), kc = c % (p / 8);
+    crow[j] = r;
+    ccol[j] = (blk + m2 * (nb / 2)) * p + kc * 8;
+    clds[j] = (m2 * 32 + r) * AROW + kc * 8;
+  });
+  u32x4 ra[NCH];
+  auto gload = [&](int m0) __attribute__((always_inline)) {
+    static_for<0, NCH>([&](auto jj_) {
+      constexpr int j = decltype(jj_)::value;
+      int row = m0 + crow[j];
+      row = row < M ? row : M - 1;
+      ra[j] = *reinterpret_cast<const u32x4*>(x + (long)row * in_f + ccol[j]);
+    });
+  };
+  auto sstore = [&](int buf) __attribute__((always_inline)) {
+    static_for<0, NCH>([&](auto jj_) {
+      *reinterpret_cast<u32x4*>(sA + buf * ABUF + clds[decltype(jj_)::value]) = ra[decltype(jj_)::value];
+    });
+  };
+  auto store_tile = [&](int buf, int m0) __attribute__((always_inline)) {
+    static_for<0, 32 * (NC / 8) / NT>([&](auto jj_) {       // 32 rows x NC / 8 pieces of 16 bytes
+      const int id = tid + NT * decltype(jj_)::value, r = id / (NC / 8), c = id % (NC / 8);
+      const u32x4 v = *reinterpret_cast<const u32x4*>(sG + (buf * 32 + r) * GROW + 8 * c);
+      if (m0 + r < M) *reinterpret_cast<u32x4*>(out + (long)(m0 + r) * I + n0 + 8 * c) = v;
+    });
+  };
+  auto product = [&](int buf, floatx16& accg, floatx16& accv) __attribute__((always_inline)) {
+    const uint16_t* ag = sA + buf * ABUF + i32 * AROW + 8 * half;
+    const uint16_t* av = ag + 32 * AROW;
+    static_for<0, 16>([&](auto vv) { accg[decltype(vv)::value] = 0.f; accv[decltype(vv)::value] = 0.f; });
+    static_for<0, KS>([&](auto kk) {
+      constexpr int ks = decltype(kk)::value;
+      accg = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(ag + 16 * ks), bwg[ks], accg, 0, 0, 0);
+      accv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(av + 16 * ks), bwv[ks], accv, 0, 0, 0);
+    });
+  };
+  // accumulator element v: row 8 (v / 4) + 4 half + v % 4, column 32 wave + i32
+  auto epilogue = [&](int buf, const floatx16& accg, const floatx16& accv) __attribute__((always_inline)) {
+    uint16_t* gt = sG + (buf * 32 + 4 * half) * GROW + 32 * wave + i32;
+    static_for<0, 8>([&](auto vv) {
+      constexpr int v = 2 * decltype(vv)::value;
+      const uint32_t pk = pack_bf16x2(gelu_erf(accg[v]) * accv[v], gelu_erf(accg[v + 1]) * accv[v + 1]);
+      gt[(8 * (v >> 2) + (v & 3)) * GROW] = (uint16_t)pk;
+      gt[(8 * (v >> 2) + (v & 3) + 1) * GROW] = (uint16_t)(pk >> 16);
+    });
+  };
+
+  floatx16 g0, v0, g1, v1;
+  gload(m_begin);
+  sstore(0);
+  if (nslab > 1) gload(m_begin + 32);
+  __syncthreads();
+  product(0, g0, v0);
+  if (nslab > 1) {
+    sstore(1);
+    if (nslab > 2) gload(m_begin + 64);
+  }
+  // step s: the product of slab s + 1 and the epilogue of slab s in one basic block; tile s - 1 goes to global memory
+  auto step = [&](int s, floatx16& ga, floatx16& va, floatx16& gb, floatx16& vb) __attribute__((always_inline)) {
+    __syncthreads();      // slab s + 1 is in sA[(s + 1) & 1]; tile s - 1 is complete in sG[(s - 1) & 1]
+    if (s > 0) store_tile((s - 1) & 1, m_begin + 32 * (s - 1));
+    product((s + 1) & 1, gb, vb);
+    epilogue(s & 1, ga, va);
+    // issue order inside this block: one MFMA, its next operand read, then a share of the epilogue's vector ALU
+    // work (about 9 instructions per MFMA) and LDS writes, so that the two pipes run side by side
+    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);      // operand reads run six MFMAs ahead
+    static_for<0, 2 * KS>([&](auto) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, (216 + 2 * KS - 1) / (2 * KS), 0);
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    });
+    if (s + 2 < nslab) {
+      sstore(s & 1);                           // last read by the product of slab s, before this step's barrier
+      if (s + 3 < nslab) gload(m_begin + 32 * (s + 3));
+    }
+  };
+  auto last_step = [&](int s, floatx16& ga, floatx16& va) __attribute__((always_inline)) {
+    __syncthreads();
+    if (s > 0) store_tile((s - 1) & 1, m_begin + 32 * (s - 1));
+    epilogue(s & 1, ga, va);
+  };
+  int s = 0;
+  for (; s + 2 < nslab; s += 2) {
+    step(s, g0, v0, g1, v1);
+    step(s + 1, g1, v1, g0, v0);
+  }
+  if (s + 1 < nslab) {
+    step(s, g0, v0, g1, v1);
+    last_step(s + 1, g1, v1);
+  } else {
+    last_step(s, g0, v0);
+  }
+  __syncthreads();
+  store_tile((nslab - 1) & 1, m_begin + 32 * (nslab - 1));
+}
+
 template <int KS>
 static int launch_glu_ws(const void* x, const void* w, void* out, int M, int nb, int q, hipStream_t stream) {
   constexpr int p = 16 * KS;
-  const size_t lds = ((size_t)2 * 2 * 32 * (p + 8) + (size_t)2 * 32 * (128 + 8)) * sizeof(uint16_t);
-  auto kern = blockdiag_glu_ws_kernel<KS>;
+  constexpr bool PIPELINED = KS <= 12;      // beyond that the second accumulator set does not fit the registers
+  const int I = nb * q / 2;
+  constexpr int NW = PIPELINED ? 8 : 4;
+  const bool wide = PIPELINED && q % (32 * NW) == 0;
+  const int ncols = wide ? 32 * NW : 128;
+  // dynamic LDS: the A slabs, and for the plain kernel the result tiles too (the pipelined one declares them itself)
+  const size_t lds = ((size_t)2 * 2 * 32 * (p + 8) + (PIPELINED ? 0 : (size_t)2 * 32 * (128 + 8))) * sizeof(uint16_t);
+  auto kern = !PIPELINED ? blockdiag_glu_ws_kernel<KS> : wide ? blockdiag_glu_ws3_kernel<KS, NW> : blockdiag_glu_ws3_kernel<KS, 4>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(blockdiag_glu_ws): %s", hipGetErrorString(e));
   }
-  const int I = nb * q / 2, nslices = I / 128;
-  // rows per workgroup: long runs amortise the weight load, but keep at least ~4 workgroups per CU
+  const int nslices = I / ncols;
+  // rows per workgroup: long runs amortise the weight load, but keep at least ~3 workgroups per CU
   int rows = 512;
-  while (rows > 128 && (long)nslices * ((M + rows - 1) / rows) < 4L * num_cus()) rows >>= 1;
+  while (rows > 128 && (long)nslices * ((M + rows - 1) / rows) < 3L * num_cus()) rows >>= 1;
   const int nchunks = (M + rows - 1) / rows;
-  hipLaunchKernelGGL(kern, dim3(nslices * nchunks), dim3(256), lds, stream, (const uint16_t*)x,
+  hipLaunchKernelGGL(kern, dim3(nslices * nchunks), dim3(wide ? 64 * NW : 256), lds, stream, (const uint16_t*)x,
                      (const uint16_t*)w, (uint16_t*)out, M, nb, q, rows);
   return check_launch("blockdiag_glu_ws");
 }
