@@ -246,6 +246,220 @@ static int launch_blockdiag(const void* x, const void* w, const float* bias, con
   return check_launch("blockdiag");
 }
 
+// ---------------------------------------------------------------------------------------------
+// Block-diagonal linear layer with a 256 x 192 workgroup tile (q a multiple of 192: d = 768, 1536).
+//
+// Operand delivery (L2 -> LDS -> registers) bounds these GEMMs long before the MFMA pipe does, so the tile is
+// as large as the register file allows: 8 waves as 4 (row groups of 64) x 2 (column halves of 96), 6 MFMA
+// tiles = 96 accumulators per lane, and with q = 192 a tile spans the whole width of a block, so every x
+// element is fetched exactly once.  K advances in chunks of 64 through a double-buffered LDS stage (one
+// barrier per chunk, the chunk after next in flight in registers); per K step of 16 a wave reads 2 A and 3 B
+// operands for 6 MFMAs.  Epilogue: bias + bf16 residual, rows leave through LDS 64 at a time as full segments.
+// ---------------------------------------------------------------------------------------------
+constexpr int kWideBN = 192;
+// WRG = row groups of 64: 4 (256 rows, 8 waves, one workgroup per compute unit, double-buffered LDS and two chunks
+// in flight in registers) or 2 (128 rows, 4 waves, one LDS stage, so that two workgroups share a compute unit and
+// one's epilogue overlaps the other's main loop).
+template <typename OUT, int WRG>
+__global__ __launch_bounds__(128 * WRG) __attribute__((amdgpu_waves_per_eu(2, 2))) void blockdiag_wide_kernel(
+    const uint16_t* __restrict__ x,      // (M, nb p) bf16
+    const uint16_t* __restrict__ w,      // (nb, q, p) bf16
+    const float* __restrict__ bias,      // (nb q) or null
+    const uint16_t* __restrict__ resid,  // (M, nb q) bf16 or null
+    OUT* __restrict__ out,               // (M, nb q)
+    int M, int nb, int p, int q) {
+  constexpr int BM = 64 * WRG, BN = kWideBN, NT = 128 * WRG;
+  constexpr bool TWO_STAGE = WRG == 4;
+  constexpr int A_CH = BM * (kBK / 8) / NT, B_CH = BN * (kBK / 8) / NT;        // chunks of 16 bytes per thread: 4 and 3 or 6
+  constexpr int STAGE = (BM + BN) * kLdsRow;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
+  const int wr = wave >> 1, wc = wave & 1;
+  int tile_m, tile_n;
+  {
+    const int ntm = (M + BM - 1) / BM, ntn = nb * q / BN;
+    const int id = blockIdx.x, e = id & 7, l = id >> 3;
+    const int full = (ntm / 8) * 8;
+    if (id < full * ntn) { tile_m = (l / ntn) * 8 + e; tile_n = l % ntn; }
+    else { const int rid = id - full * ntn; tile_m = full + rid / ntn; tile_n = rid % ntn; }
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int in_f = nb * p, out_cols = nb * q;
+  const int blk = n0 / q, jj = n0 % q;
+  const int nchunks = p / kBK;
+
+  const uint16_t* pa[A_CH];
+  const uint16_t* pb[B_CH];
+  int la[A_CH], lb[B_CH];
+  static_for<0, A_CH>([&](auto jj_) {
+    constexpr int j = decltype(jj_)::value;
+    const int id = tid + NT * j, r = id >> 3, kc = id & 7;
+    int row = m0 + r;
+    row = row < M ? row : M - 1;
+    pa[j] = x + (long)row * in_f + (long)blk * p + kc * 8;
+    la[j] = r * kLdsRow + kc * 8;
+  });
+  static_for<0, B_CH>([&](auto jj_) {
+    constexpr int j = decltype(jj_)::value;
+    const int id = tid + NT * j, r = id >> 3, kc = id & 7;
+    pb[j] = w + ((long)blk * q + jj + r) * p + kc * 8;
+    lb[j] = (BM + r) * kLdsRow + kc * 8;
+  });
+  // two chunks in flight in registers (ring slot = chunk & 1) on top of the one waiting in the other LDS stage:
+  // with one workgroup per compute unit the loads in flight are what hides the memory latency
+  u32x4 ra[TWO_STAGE ? 2 : 1][A_CH], rb[TWO_STAGE ? 2 : 1][B_CH];
+  auto gload = [&](int c, auto slot_) __attribute__((always_inline)) {
+    constexpr int sl = decltype(slot_)::value;
+    static_for<0, A_CH>([&](auto jj_) { ra[sl][decltype(jj_)::value] = *reinterpret_cast<const u32x4*>(pa[decltype(jj_)::value] + c * kBK); });
+    static_for<0, B_CH>([&](auto jj_) { rb[sl][decltype(jj_)::value] = *reinterpret_cast<const u32x4*>(pb[decltype(jj_)::value] + c * kBK); });
+  };
+  auto sstore = [&](int stage, auto slot_) __attribute__((always_inline)) {
+    constexpr int sl = decltype(slot_)::value;
+    uint16_t* st = smem + stage * STAGE;
+    static_for<0, A_CH>([&](auto jj_) { *reinterpret_cast<u32x4*>(st + la[decltype(jj_)::value]) = ra[sl][decltype(jj_)::value]; });
+    static_for<0, B_CH>([&](auto jj_) { *reinterpret_cast<u32x4*>(st + lb[decltype(jj_)::value]) = rb[sl][decltype(jj_)::value]; });
+  };
+
+  floatx16 acc[2][3];
+  static_for<0, 6>([&](auto tt) {
+    static_for<0, 16>([&](auto vv) { acc[decltype(tt)::value / 3][decltype(tt)::value % 3][decltype(vv)::value] = 0.f; });
+  });
+  auto compute = [&](int stage) __attribute__((always_inline)) {
+    const uint16_t* sa = smem + stage * STAGE + (wr * 64 + i32) * kLdsRow + 8 * half;
+    const uint16_t* sb = smem + stage * STAGE + (BM + wc * 96 + i32) * kLdsRow + 8 * half;
+    static_for<0, kBK / 16>([&](auto kk_) {
+      constexpr int kk = decltype(kk_)::value;
+      bf16x8 av[2], bv[3];
+      av[0] = ld8(sa + kk * 16);
+      av[1] = ld8(sa + 32 * kLdsRow + kk * 16);
+      static_for<0, 3>([&](auto bb) { bv[decltype(bb)::value] = ld8(sb + 32 * decltype(bb)::value * kLdsRow + kk * 16); });
+      static_for<0, 6>([&](auto tt) {
+        constexpr int a = decltype(tt)::value / 3, b = decltype(tt)::value % 3;
+        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[a], bv[b], acc[a][b], 0, 0, 0);
+      });
+    });
+  };
+  if constexpr (TWO_STAGE) {
+    // chunk c is multiplied from LDS stage c & 1 while chunk c + 1 moves from ring slot (c + 1) & 1 to the other
+    // stage and chunk c + 3 is requested into that slot
+    auto step = [&](int c, auto par_) __attribute__((always_inline)) {
+      constexpr int nx = (decltype(par_)::value + 1) & 1;          // (c + 1) & 1
+      compute(c & 1);
+      if (c + 1 < nchunks) {
+        sstore(nx, ic<nx>{});                // that stage was last read before the barrier that ended chunk c - 1
+        if (c + 3 < nchunks) gload(c + 3, ic<nx>{});
+      }
+      __syncthreads();
+    };
+    gload(0, ic<0>{});
+    sstore(0, ic<0>{});
+    if (nchunks > 1) gload(1, ic<1>{});
+    if (nchunks > 2) gload(2, ic<0>{});
+    __syncthreads();
+    int c = 0;
+    for (; c + 1 < nchunks; c += 2) {
+      step(c, ic<0>{});
+      step(c + 1, ic<1>{});
+    }
+    if (c < nchunks) step(c, ic<0>{});
+  } else {
+    // one LDS stage: the next chunk waits in registers while this one is multiplied (two barriers per chunk)
+    gload(0, ic<0>{});
+    sstore(0, ic<0>{});
+    if (nchunks > 1) gload(1, ic<0>{});
+    __syncthreads();
+    for (int c = 0; c < nchunks; ++c) {
+      compute(0);
+      __syncthreads();
+      if (c + 1 < nchunks) {
+        sstore(0, ic<0>{});
+        if (c + 2 < nchunks) gload(c + 2, ic<0>{});
+      }
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue: 64 rows at a time (the rows of wave row group ep) through an fp32 LDS tile.  The residual
+  // values of a pass are requested one pass ahead, all at once: loaded where they are used, every row of the
+  // copy loop waited a full memory latency ----
+  constexpr int OROW = BN + 4;
+  constexpr int TPR = BN / 4, RPI = NT / TPR;           // 48 threads per row: 10 or 5 rows per sweep
+  constexpr int NR = (64 + RPI - 1) / RPI;              // rows per thread and pass: 7 or 13
+  float* so_base = reinterpret_cast<float*>(smem);
+  const int cq = (tid % TPR) * 4, r0 = tid / TPR;
+  float4 bq = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (bias) bq = *reinterpret_cast<const float4*>(bias + n0 + cq);
+  auto row_ok = [&](int ep, int i) { return tid < TPR * RPI && r0 + i * RPI < 64 && m0 + ep * 64 + r0 + i * RPI < M; };
+  uint32_t rx[2][NR], ry[2][NR];
+  auto load_resid = [&](int ep, auto slot_) __attribute__((always_inline)) {
+    constexpr int sl = decltype(slot_)::value;
+    static_for<0, NR>([&](auto ii) {
+      constexpr int i = decltype(ii)::value;
+      uint2 rr = make_uint2(0u, 0u);
+      if (resid && row_ok(ep, i))
+        rr = *reinterpret_cast<const uint2*>(resid + (long)(m0 + ep * 64 + r0 + i * RPI) * out_cols + n0 + cq);
+      rx[sl][i] = rr.x;
+      ry[sl][i] = rr.y;
+    });
+  };
+  load_resid(0, ic<0>{});
+  static_for<0, WRG>([&](auto ee) {
+    constexpr int ep = decltype(ee)::value, sl = ep & 1;
+    if (wr == ep) {
+      float* so = so_base + (4 * half) * OROW + wc * 96 + i32;
+      static_for<0, 6>([&](auto tt) {
+        constexpr int a = decltype(tt)::value / 3, b = decltype(tt)::value % 3;
+        static_for<0, 16>([&](auto vv) {
+          constexpr int v = decltype(vv)::value;
+          so[(32 * a + 8 * (v >> 2) + (v & 3)) * OROW + 32 * b] = acc[a][b][v];
+        });
+      });
+    }
+    if constexpr (ep + 1 < WRG) load_resid(ep + 1, ic<(sl ^ 1)>{});
+    __syncthreads();
+    static_for<0, NR>([&](auto ii) {
+      constexpr int i = decltype(ii)::value;
+      if (row_ok(ep, i)) {
+        const int r = r0 + i * RPI;
+        float4 v4 = *reinterpret_cast<const float4*>(so_base + r * OROW + cq);
+        const long o = (long)(m0 + ep * 64 + r) * out_cols + n0 + cq;
+        v4.x += bq.x + __uint_as_float(rx[sl][i] << 16); v4.y += bq.y + __uint_as_float(rx[sl][i] & 0xffff0000u);
+        v4.z += bq.z + __uint_as_float(ry[sl][i] << 16); v4.w += bq.w + __uint_as_float(ry[sl][i] & 0xffff0000u);
+        if constexpr (sizeof(OUT) == 2) {
+          uint2 pk;
+          pk.x = pack_bf16x2(v4.x, v4.y);
+          pk.y = pack_bf16x2(v4.z, v4.w);
+          *reinterpret_cast<uint2*>(out + o) = pk;
+        } else {
+          *reinterpret_cast<float4*>(out + o) = v4;
+        }
+      }
+    });
+    __syncthreads();
+  });
+}
+
+template <typename OUT>
+static int launch_blockdiag_wide(const void* x, const void* w, const float* bias, const void* resid, void* out, int M,
+                                 int nb, int p, int q, hipStream_t stream) {
+  // 128-row tiles (two workgroups per compute unit) once there are enough of them to fill the chip twice over
+  const bool small = (long)((M + 127) / 128) * (nb * q / kWideBN) >= 4L * num_cus();
+  const int bm = small ? 128 : 256;
+  const size_t stage = (size_t)(bm + kWideBN) * kLdsRow * sizeof(uint16_t);
+  const size_t epi = (size_t)64 * (kWideBN + 4) * sizeof(float);
+  size_t lds = small ? stage : 2 * stage;
+  if (lds < epi) lds = epi;
+  auto kern = small ? blockdiag_wide_kernel<OUT, 2> : blockdiag_wide_kernel<OUT, 4>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(blockdiag_wide): %s", hipGetErrorString(e));
+  }
+  dim3 grid(((M + bm - 1) / bm) * (nb * q / kWideBN));
+  hipLaunchKernelGGL(kern, grid, dim3(2 * bm), lds, stream, (const uint16_t*)x, (const uint16_t*)w, bias,
+                     (const uint16_t*)resid, (OUT*)out, M, nb, p, q);
+  return check_launch("blockdiag_wide");
+}
+
 // LayerNorm over the last dimension of x (M, d) fp32, eps inside the square root.
 // Workgroup = 8 waves handles R = 8 RW rows; each wave normalises RW rows at once (all loads in flight
 // together) and writes the row-major outputs from registers.  For the channel-major output the
@@ -718,6 +932,9 @@ extern "C" int m2_blockdiag_linear_fwd(const void* x, const void* w, const float
   int rc = check_blockdiag("m2_blockdiag_linear_fwd", M, nblocks, p, q, false);
   if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
+  if (q % kWideBN == 0)
+    return out_dtype == M2_DTYPE_F32 ? launch_blockdiag_wide<float>(x, w, bias, residual, out, M, nblocks, p, q, st)
+                                     : launch_blockdiag_wide<uint16_t>(x, w, bias, residual, out, M, nblocks, p, q, st);
   const bool wide = q % 128 == 0;
   if (out_dtype == M2_DTYPE_F32)
     return wide ? launch_blockdiag<2, 2, false, float, 1>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st)

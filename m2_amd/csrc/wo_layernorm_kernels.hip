@@ -139,12 +139,22 @@ __global__ __launch_bounds__(512) void wo_layernorm_kernel(
   float* red = reinterpret_cast<float*>(lds_raw + TILE_BYTES);               // [2][NB][64]
   if (resid) {
     constexpr int PPR = D / 8;                                               // 16-byte pieces per row
-    for (int id = tid; id < kWBM * PPR; id += 512) {
-      const int r = id / PPR, pc = id % PPR;
+    constexpr int NP = kWBM * PPR / 512;                                     // pieces per thread: 12 at d = 768
+    static_assert(kWBM * PPR % 512 == 0, "residual tile must divide over the threads");
+    // all loads first, then all LDS stores: one memory latency for the tile, not one per piece
+    u32x4 rr[NP];
+    static_for<0, NP>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      const int id = tid + 512 * j, r = id / PPR, pc = id % PPR;
       int row = m0 + r;
       row = row < M ? row : M - 1;
-      *reinterpret_cast<u32x4*>(sR + r * S::RROW + 8 * pc) = *reinterpret_cast<const u32x4*>(resid + (long)row * D + 8 * pc);
-    }
+      rr[j] = *reinterpret_cast<const u32x4*>(resid + (long)row * D + 8 * pc);
+    });
+    static_for<0, NP>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      const int id = tid + 512 * j, r = id / PPR, pc = id % PPR;
+      *reinterpret_cast<u32x4*>(sR + r * S::RROW + 8 * pc) = rr[j];
+    });
     __syncthreads();
   }
   float gm[QT], bt[QT];

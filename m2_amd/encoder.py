@@ -117,6 +117,11 @@ class BertGatedLinearUnitMLP(nn.Module):
         self.dropout = nn.Dropout(config.hidden_dropout_prob)
         self.layernorm = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_eps)
 
+    # True: wo + bias + residual + LayerNorm as one kernel (d <= 768).  Off by default: the 256 x 192-tile wo
+    # kernel followed by the LayerNorm kernel measured faster on MI355X (9.06 against 9.13 ms per forward at
+    # L = 8192, B = 4; 2.00 against 2.24 ms at L = 128, B = 32), although it writes and re-reads the fp32 sum.
+    fuse_wo_layernorm = False
+
     def presum(self, a16: torch.Tensor) -> torch.Tensor:
         """a16 (M, d) bf16 -> wo(glu(a16)) + bias + a16, (M, d) fp32 (the LayerNorm input)."""
         g = ops.blockdiag_glu(a16, self.gated_layers.weight_bf16())
@@ -128,11 +133,12 @@ class BertGatedLinearUnitMLP(nn.Module):
 
     def normed(self, a16: torch.Tensor, want_f32: bool, want_bf16: bool, want_channel_major: bool):
         """a16 (M, d) bf16 -> LayerNorm(wo(glu(a16)) + bias + a16) in the requested forms (f32 | None, bf16 | None,
-        channel-major f32 | None).  `wo` and the LayerNorm are one kernel where the shape allows it."""
+        channel-major f32 | None).  With `fuse_wo_layernorm`, `wo` and the LayerNorm are one kernel where the shape
+        allows it."""
         gamma, beta, eps = self.ln_params()
         w = self.wo.weight_bf16()
         nb, q, p = w.shape
-        if ops.blockdiag_linear_layernorm_supported(nb * p, nb * q, nb):
+        if self.fuse_wo_layernorm and ops.blockdiag_linear_layernorm_supported(nb * p, nb * q, nb):
             g = ops.blockdiag_glu(a16, self.gated_layers.weight_bf16())
             return ops.blockdiag_linear_layernorm(g, w, self.wo.bias.detach().float().contiguous(), a16, gamma, beta, eps,
                                                   want_f32=want_f32, want_bf16=want_bf16,

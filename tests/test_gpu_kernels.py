@@ -125,6 +125,24 @@ def test_blockdiag_glu_and_linear(gpu, M, d, I):
     assert rel_err(got3.float(), O.blockdiag_multiply(a.double(), wo.double()))[0] < TOL_BF16
 
 
+def test_blockdiag_linear_full_size_ragged(gpu):
+    """wo at the benchmark's M with a ragged last tile (the shape that selects the 128-row tiles, two workgroups
+    per compute unit), bias + bf16 residual, fp32 and bf16 outputs; fp32 oracle on the CPU."""
+    from m2_amd import ops
+    from oracle import m2_oracle as O
+    M, d, I, nb = 32768 - 70, 768, 3072, 4
+    g = torch.Generator().manual_seed(21)
+    a = torch.randn(M, I, generator=g).bfloat16()
+    wo = (torch.randn(nb, d // nb, I // nb, generator=g) * 0.05).bfloat16()
+    bias = torch.randn(d, generator=g)
+    res = torch.randn(M, d, generator=g).bfloat16()
+    ref = O.blockdiag_multiply(a.float(), wo.float()) + bias + res.float()
+    got = ops.blockdiag_linear(a.to(gpu), wo.to(gpu), bias.to(gpu), res.to(gpu), out_dtype=torch.float32)
+    assert rel_err(got, ref)[0] < 1e-3
+    got16 = ops.blockdiag_linear(a.to(gpu), wo.to(gpu), bias.to(gpu), res.to(gpu), out_dtype=torch.bfloat16)
+    assert rel_err(got16.float(), ref)[0] < TOL_BF16
+
+
 @pytest.mark.parametrize("M,d", [(300, 768), (64, 1536), (1000, 128)])
 def test_layernorm_three_outputs(gpu, M, d):
     from m2_amd import ops
@@ -179,6 +197,12 @@ def test_encoder_small(gpu, L, B, layers):
     for layer in model.encoder.layer:
         x = layer(x)
     e, e2 = rel_err(x, ref)
+    assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
+    # wo + LayerNorm as one kernel (an option; two kernels are the default)
+    for layer in model.encoder.layer:
+        layer.mlp.fuse_wo_layernorm = True
+    out1, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
+    e, e2 = rel_err(out1, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
 
 
