@@ -200,30 +200,42 @@ __global__ __launch_bounds__(256) void blockdiag_kernel(
         });
       });
     }
+    // the residual values of the pass are requested all at once, before the barrier: loaded where they are used,
+    // every row of the copy loop waited a full memory latency
+    constexpr int NR = EROWS / RPI;
+    static_assert(EROWS % RPI == 0, "rows of a pass must divide over the threads");
+    uint2 rres[NR];
+    if constexpr (!GLU) {
+      static_for<0, NR>([&](auto ii) {
+        constexpr int i = decltype(ii)::value;
+        const int row = m0 + ep * EROWS + tid / TPR + i * RPI;
+        rres[i] = make_uint2(0u, 0u);
+        if (resid && row < M) rres[i] = *reinterpret_cast<const uint2*>(resid + (long)row * out_cols + n0 + cq);
+      });
+    }
     __syncthreads();
     const float* srow = reinterpret_cast<const float*>(smem) + cq;
-    for (int r = tid / TPR; r < EROWS; r += RPI) {
+    static_for<0, NR>([&](auto ii) {
+      constexpr int i = decltype(ii)::value;
+      const int r = tid / TPR + i * RPI;
       const int row = m0 + ep * EROWS + r;
-      if (row >= M) break;
-      float4 v4 = *reinterpret_cast<const float4*>(srow + r * OROW);
-      const long o = (long)row * out_cols + n0 + cq;
-      if constexpr (!GLU) {
-        v4.x += bq.x; v4.y += bq.y; v4.z += bq.z; v4.w += bq.w;
-        if (resid) {
-          const uint2 rr = *reinterpret_cast<const uint2*>(resid + o);
-          v4.x += __uint_as_float(rr.x << 16); v4.y += __uint_as_float(rr.x & 0xffff0000u);
-          v4.z += __uint_as_float(rr.y << 16); v4.w += __uint_as_float(rr.y & 0xffff0000u);
+      if (row < M) {
+        float4 v4 = *reinterpret_cast<const float4*>(srow + r * OROW);
+        const long o = (long)row * out_cols + n0 + cq;
+        if constexpr (!GLU) {
+          v4.x += bq.x + __uint_as_float(rres[i].x << 16); v4.y += bq.y + __uint_as_float(rres[i].x & 0xffff0000u);
+          v4.z += bq.z + __uint_as_float(rres[i].y << 16); v4.w += bq.w + __uint_as_float(rres[i].y & 0xffff0000u);
+        }
+        if constexpr (sizeof(OUT) == 2) {
+          uint2 pk;
+          pk.x = pack_bf16x2(v4.x, v4.y);
+          pk.y = pack_bf16x2(v4.z, v4.w);
+          *reinterpret_cast<uint2*>(out + o) = pk;
+        } else {
+          *reinterpret_cast<float4*>(out + o) = v4;
         }
       }
-      if constexpr (sizeof(OUT) == 2) {
-        uint2 pk;
-        pk.x = pack_bf16x2(v4.x, v4.y);
-        pk.y = pack_bf16x2(v4.z, v4.w);
-        *reinterpret_cast<uint2*>(out + o) = pk;
-      } else {
-        *reinterpret_cast<float4*>(out + o) = v4;
-      }
-    }
+    });
     if (ep + 1 < EP) __syncthreads();
   }
 }
