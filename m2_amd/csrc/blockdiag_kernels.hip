@@ -3,10 +3,12 @@
 //
 //   out[m, k q + j] = sum_i x[m, k p + i] w[k, j, i]          (bert/src/mm/blockdiag_multiply.py:19-34,49-60)
 //
-// `blockdiag_kernel<GLU=true>`  computes gelu_erf(gate) * value in the epilogue, where gate column j
-// (block j / q) pairs with value column I + j (block j / q + nb/2)   (bert/src/bert_layers.py:482-502).
-// `blockdiag_kernel<GLU=false>` adds bias and a residual                (bert/src/bert_layers.py:504-506,
-//                                                                        bert/src/mm/structured_linear.py:65-69).
+// Gated form: gelu_erf(gate) * value in the epilogue, where gate column j (block j / q) pairs with value
+// column I + j (block j / q + nb/2)   (bert/src/bert_layers.py:482-502): `blockdiag_glu_ws3_kernel` (K <= 192,
+// weights stationary in registers, software-pipelined), `blockdiag_glu_ws_kernel` (K = 256),
+// `blockdiag_kernel<GLU=true>` (longer K).
+// Plain form with bias and a residual (bert/src/bert_layers.py:504-506, bert/src/mm/structured_linear.py:65-69):
+// `blockdiag_wide_kernel` (192-column tiles: q a multiple of 192), `blockdiag_kernel<GLU=false>` (other widths).
 // `layernorm_kernel` normalises rows and writes the three forms the next layer reads.
 //
 // MFMA: v_mfma_f32_32x32x16_bf16.  Lane (i = lane % 32, h = lane / 32) supplies A[i][8h .. 8h+7] and

@@ -155,22 +155,24 @@ __device__ __forceinline__ int slot_of(int t, int i, int j) { return t + P::T * 
 
 // Causal 3-tap convolution of one (3d, B, L) channel at the time steps of this thread's 32 slots:
 // out[r] = (sc(2m), sc(2m+1)) with sc(n) = bias + w0 in[n-2] + w1 in[n-1] + w2 in[n], in = stored value + add
-// (time steps before 0 are the convolution's zero padding).  The 64 loads are put in flight in two batches.
+// (time steps before 0 are the convolution's zero padding).  All 64 loads of a bf16 row are put in flight at once
+// (64 registers); an fp32 row goes in two batches.
 template <class P, typename ACT>
 __device__ __forceinline__ void short_conv_slots(const ACT* __restrict__ p, int t, const float (&w)[3], float bias,
                                                  float add, cf (&out)[32]) {
   typedef typename PairBits<ACT>::type bits;
-  static_for<0, 2>([&](auto hh) {
-    constexpr int h0 = decltype(hh)::value * 16;
-    bits prev[16], cur[16];
-    static_for<0, 16>([&](auto rr) {
+  constexpr int NB = sizeof(ACT) == 2 ? 32 : 16;      // slots per batch
+  static_for<0, 32 / NB>([&](auto hh) {
+    constexpr int h0 = decltype(hh)::value * NB;
+    bits prev[NB], cur[NB];
+    static_for<0, NB>([&](auto rr) {
       constexpr int r = h0 + decltype(rr)::value;
       const int m = slot_of<P>(t, r / P::R1, r % P::R1);
       cur[r - h0] = fetch_pair(p, m);
       prev[r - h0] = fetch_pair(p, m - 1);
     });
     __builtin_amdgcn_sched_barrier(0);
-    static_for<0, 16>([&](auto rr) {
+    static_for<0, NB>([&](auto rr) {
       constexpr int r = h0 + decltype(rr)::value;
       const int m = slot_of<P>(t, r / P::R1, r % P::R1);
       float2 c = expand_pair(cur[r - h0]), q = expand_pair(prev[r - h0]);
