@@ -207,6 +207,8 @@ class BertEncoder(nn.Module):
     cached bf16 copies): it is dropped by `load_state_dict`, `.to()` / `.cuda()` and `reset_graphs()`; call
     `reset_graphs()` after changing a parameter in place.  Nothing in the captured region uses a memset."""
 
+    OVERLAP_UPFRONT_MAX_L = 2048
+
     def __init__(self, config: M2BertConfig, use_hip_graph: bool = False):
         super().__init__()
         self.layer = nn.ModuleList([BertLayer(config) for _ in range(config.num_hidden_layers)])
@@ -214,11 +216,16 @@ class BertEncoder(nn.Module):
         self.num_attention_heads = config.num_attention_heads
         self.use_hip_graph = use_hip_graph
         self._graphs = {}
-        # Filter generation depends on the weights only.  With overlap_filters the spectra of layer i + 1 are
-        # generated on a second stream (default priority) while layer i runs its projections and MLP, i.e.
-        # next to the memory-bound kernels and not next to the mixer core.  Off by default: at L = 8192, B = 4 it
-        # shortens the forward by about 1 % only (the GPU mostly serialises the two streams).
-        self.overlap_filters = False
+        # Filter generation depends on the weights only, so it can run on a second stream (default priority):
+        #   "upfront"  all layers' spectra one after the other from the start of the forward, each layer waiting
+        #              for its own (holds all spectra at once: 100 MB per layer at L = 8192, d = 768);
+        #   True       the spectra of layer i + 1 behind the mixer core of layer i;
+        #   False      in line, on the main stream;
+        #   None       "upfront" for sequences up to OVERLAP_UPFRONT_MAX_L, where the generation kernels are a few
+        #              workgroups each and pure latency (forward as one HIP graph at d = 768: -10 % at L = 256,
+        #              -7 % at L = 1024, -2 % at L = 2048 .. 8192), in line beyond, where concurrent kernels also
+        #              blur per-kernel timings.
+        self.overlap_filters = None
         self._filter_stream = None
 
     # -- graph bookkeeping -------------------------------------------------------------------
@@ -251,6 +258,8 @@ class BertEncoder(nn.Module):
             o32 = h32
             cur = torch.cuda.current_stream()
             overlap = self.overlap_filters
+            if overlap is None:
+                overlap = "upfront" if L <= self.OVERLAP_UPFRONT_MAX_L else False
             nxt = [None, None]                       # spectra of the next layer and the event that says they are ready
             if overlap:
                 if self._filter_stream is None:
@@ -269,12 +278,26 @@ class BertEncoder(nn.Module):
                         ev.record(side)
                     nxt[0], nxt[1] = sp, ev
 
-                generate(0, None)
+                upfront = overlap == "upfront"
+                ahead = []
+                if upfront:          # all layers' spectra at once, in order, while the main stream runs the layers
+                    side.wait_stream(cur)
+                    with torch.cuda.stream(side):
+                        for lay in self.layer:
+                            sp = lay.attention.filter_spectrum(L)
+                            sp.record_stream(cur)
+                            ev = torch.cuda.Event()
+                            ev.record(side)
+                            ahead.append((sp, ev))
+                else:
+                    generate(0, None)
             for i, layer in enumerate(self.layer):
                 want = all_layers or i == n - 1
                 keep32 = want or pre_norm
                 spec, ready, hook = None, None, None
-                if overlap:
+                if overlap and upfront:
+                    spec, ready = ahead[i]
+                elif overlap:
                     spec, ready = nxt
                     if i + 1 < n:
                         def hook(i=i):

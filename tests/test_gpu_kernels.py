@@ -266,7 +266,8 @@ def test_cached_filter_spectra_follow_the_weights(gpu):
 
 
 def test_encoder_overlapped_filter_generation_matches_sequential(gpu):
-    """Generating layer i + 1's filter spectra on a second stream while layer i runs must not change a bit."""
+    """Generating the filter spectra on a second stream (next layer's behind the mixer core, or all layers' from the
+    start) must not change a bit, eagerly or as a captured graph."""
     import m2_amd
     cfg = m2_amd.m2_bert_80m(256)
     cfg.num_hidden_layers = 3
@@ -274,12 +275,26 @@ def test_encoder_overlapped_filter_generation_matches_sequential(gpu):
     model.load_state_dict(m2_amd.seeded_state_dict(cfg, 43))
     model = model.to(gpu).eval()
     ids = torch.randint(0, cfg.vocab_size, (2, 256), generator=torch.Generator().manual_seed(10)).to(gpu)
+    model.encoder.overlap_filters = False          # in line on the main stream
     want, _ = model(ids)
-    model.encoder.overlap_filters = True
-    for _ in range(3):
-        got, _ = model(ids)
+    for mode in (True, "upfront", None):            # None picks "upfront" at this length
+        model.encoder.overlap_filters = mode
+        for _ in range(3):
+            got, _ = model(ids)
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), mode
+    # and inside a captured graph (the side stream becomes a parallel branch), replayed with eager work between
+    graphed = m2_amd.BertModel(cfg, use_hip_graph=True)
+    graphed.load_state_dict(m2_amd.seeded_state_dict(cfg, 43))
+    graphed = graphed.to(gpu).eval()
+    graphed.encoder.overlap_filters = "upfront"
+    for it in range(4):
+        ids2 = torch.randint(0, cfg.vocab_size, (2, 256), generator=torch.Generator().manual_seed(20 + it)).to(gpu)
+        model.encoder.overlap_filters = False
+        want2, _ = model(ids2)
+        got2, _ = graphed(ids2)
         torch.cuda.synchronize()
-        assert torch.equal(got, want)
+        assert torch.equal(got2, want2), it
 
 
 def test_embed_layernorm_matches_oracle(gpu):
