@@ -62,6 +62,20 @@ __device__ __forceinline__ cf unit_root(int m, int n) {
   return {c, -s};
 }
 
+// Synchronisation of the threads that share a row.  A row of up to 64 threads lies inside one wavefront
+// (rows are aligned runs of T threads, T a power of two): its LDS instructions execute in program order, so a
+// later read by any lane sees an earlier write by any other lane and only the compiler has to be kept from
+// reordering them.  Longer rows need the workgroup barrier.
+template <class P>
+__device__ __forceinline__ void row_sync() {
+  if constexpr (P::T <= 64) {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  } else {
+    __syncthreads();
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // generic passes on the row held in LDS
 // ------------------------------------------------------------------------------------------
@@ -236,14 +250,14 @@ __device__ __forceinline__ void paired_groups(int w, int& g, int& g2) {
 template <class P, bool ZERO_UPPER>
 __device__ __forceinline__ void forward_to_pairs(cf (&x)[16], int t, float2* row, const Twiddles<P>& tw, int g, int g2) {
   fwd_compute_store<P, 1, P::R1, P::S1, ZERO_UPPER>(x, t, row, tw);
-  __syncthreads();
+  row_sync<P>();
   fwd_load<P, P::R2, P::S2>(x, t, row);
   fwd_compute_store<P, 2, P::R2, P::S2, false>(x, t, row, tw);
-  __syncthreads();
+  row_sync<P>();
   if constexpr (P::R3 > 1) {
     fwd_load<P, P::R3, P::S3>(x, t, row);
     fwd_compute_store<P, 3, P::R3, P::S3, false>(x, t, row, tw);
-    __syncthreads();
+    row_sync<P>();
   }
   {
     const float2* pa = row + phys(g * 8);
@@ -285,15 +299,15 @@ __device__ __forceinline__ void inverse_from_pairs(cf (&x)[16], int t, float2* r
       lds_put(pb, j, x[8 + j]);
     });
   }
-  __syncthreads();
+  row_sync<P>();
   if constexpr (P::R3 > 1) {
     inv_load_compute<P, 3, P::R3, P::S3, false>(x, t, row, tw);
     inv_store<P, P::R3, P::S3>(x, t, row);
-    __syncthreads();
+    row_sync<P>();
   }
   inv_load_compute<P, 2, P::R2, P::S2, false>(x, t, row, tw);
   inv_store<P, P::R2, P::S2>(x, t, row);
-  __syncthreads();
+  row_sync<P>();
   inv_load_compute<P, 1, P::R1, P::S1, LOWER_ONLY>(x, t, row, tw);
 }
 

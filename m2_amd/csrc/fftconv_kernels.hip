@@ -102,50 +102,55 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
     const int jj = valid ? j : rows_per_xcd - 1;
     const int c = (jj / B) * 8 + xcd, b = jj % B;
 
-    // ---- prologue: 8 consecutive time steps per thread: short conv, gate, stage z = a + i u in LDS ----
+    // ---- prologue: 8 consecutive time steps per thread: short conv, gate, stage z = a + i u in LDS.  All loads of
+    // the row are put in flight before the first is converted (one memory latency per row, not one per signal) ----
     float gate[8];
     {
       float in[10], a[8];
+      RawRow<ACT, 1> r1, r2, rv;
+      f32x4_t u0 = {0.f, 0.f, 0.f, 0.f}, u1 = u0;
+      if (sw) {
+        r1.template fetch<0>(xproj + ((long)(0 * d + c) * B + b) * L, n0);
+        rv.template fetch<0>(xproj + ((long)(2 * d + c) * B + b) * L, n0);
+        r2.template fetch<0>(xproj + ((long)(1 * d + c) * B + b) * L, n0);
+      } else {
+        r1.template fetch<0>(xproj + ((long)c * B + b) * L, n0);
+      }
+      if (uin) {
+        const float* pu = uin + ((long)c * B + b) * L + n0;
+        u0 = *reinterpret_cast<const f32x4_t*>(pu);
+        u1 = *reinterpret_cast<const f32x4_t*>(pu + 4);
+      }
       if (sw) {
         const float* w = sw + (long)c * 3;
-        load10(xproj + ((long)(0 * d + c) * B + b) * L, n0, pbias ? pbias[c] : 0.f, in);
-        {
-          const float w0 = w[0], w1 = w[1], w2 = w[2], bb = sb[c];
-          static_for<0, 8>([&](auto jj) {
-            constexpr int j = decltype(jj)::value;
-            a[j] = bb + w0 * in[j] + w1 * in[j + 1] + w2 * in[j + 2];
-          });
-        }
-        load10(xproj + ((long)(2 * d + c) * B + b) * L, n0, pbias ? pbias[2 * d + c] : 0.f, in);
-        {
-          const float w0 = w[6 * (long)d + 0], w1 = w[6 * (long)d + 1], w2 = w[6 * (long)d + 2], bb = sb[2 * d + c];
-          static_for<0, 8>([&](auto jj) {
-            constexpr int j = decltype(jj)::value;
-            a[j] *= bb + w0 * in[j] + w1 * in[j + 1] + w2 * in[j + 2];
-          });
-        }
-        load10(xproj + ((long)(1 * d + c) * B + b) * L, n0, pbias ? pbias[d + c] : 0.f, in);
-        {
-          const float w0 = w[3 * (long)d + 0], w1 = w[3 * (long)d + 1], w2 = w[3 * (long)d + 2], bb = sb[d + c];
-          static_for<0, 8>([&](auto jj) {
-            constexpr int j = decltype(jj)::value;
-            gate[j] = bb + w0 * in[j] + w1 * in[j + 1] + w2 * in[j + 2];
-          });
-        }
+        const float w10 = w[0], w11 = w[1], w12 = w[2], bb1 = sb[c];
+        const float wv0 = w[6 * (long)d + 0], wv1 = w[6 * (long)d + 1], wv2 = w[6 * (long)d + 2], bbv = sb[2 * d + c];
+        const float w20 = w[3 * (long)d + 0], w21 = w[3 * (long)d + 1], w22 = w[3 * (long)d + 2], bb2 = sb[d + c];
+        const float p1 = pbias ? pbias[c] : 0.f, pv = pbias ? pbias[2 * d + c] : 0.f, p2 = pbias ? pbias[d + c] : 0.f;
+        __builtin_amdgcn_sched_barrier(0);
+        r1.template expand<0>(n0, p1, in);
+        static_for<0, 8>([&](auto jj) {
+          constexpr int j = decltype(jj)::value;
+          a[j] = bb1 + w10 * in[j] + w11 * in[j + 1] + w12 * in[j + 2];
+        });
+        rv.template expand<0>(n0, pv, in);
+        static_for<0, 8>([&](auto jj) {
+          constexpr int j = decltype(jj)::value;
+          a[j] *= bbv + wv0 * in[j] + wv1 * in[j + 1] + wv2 * in[j + 2];
+        });
+        r2.template expand<0>(n0, p2, in);
+        static_for<0, 8>([&](auto jj) {
+          constexpr int j = decltype(jj)::value;
+          gate[j] = bb2 + w20 * in[j] + w21 * in[j + 1] + w22 * in[j + 2];
+        });
       } else {
         // plain long convolution: xproj is a single (d, B, L) signal, no short conv, no gates
-        load10(xproj + ((long)c * B + b) * L, n0, 0.f, in);
+        r1.template expand<0>(n0, 0.f, in);
         static_for<0, 8>([&](auto jj) {
           constexpr int j = decltype(jj)::value;
           a[j] = in[j + 2];
           gate[j] = 1.f;
         });
-      }
-      float4 u0 = make_float4(0.f, 0.f, 0.f, 0.f), u1 = u0;
-      if (uin) {
-        const float* pu = uin + ((long)c * B + b) * L + n0;
-        u0 = *reinterpret_cast<const float4*>(pu);
-        u1 = *reinterpret_cast<const float4*>(pu + 4);
       }
       float4* dst = reinterpret_cast<float4*>(row + phys(n0));     // 8 consecutive slots never straddle a pad
       dst[0] = make_float4(a[0], u0.x, a[1], u0.y);
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
       dst[2] = make_float4(a[4], u1.x, a[5], u1.y);
       dst[3] = make_float4(a[6], u1.z, a[7], u1.w);
     }
-    __syncthreads();
+    row_sync<P>();
 
     cf x[16];
     fwd_load_lower<P>(x, t, row);
@@ -188,7 +193,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
     // ---- inverse ----
     inverse_from_pairs<P, true>(x, t, row, tw, g, g2);
     inv_store_lower<P>(x, t, row);      // only slots this thread has just read are overwritten
-    __syncthreads();
+    row_sync<P>();
 
     // ---- epilogue: 8 consecutive outputs per thread ----
     {
@@ -201,7 +206,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
       out[6] = o3.x * gate[6] + o3.y; out[7] = o3.z * gate[7] + o3.w;
       if (valid) store8(y + ((long)c * B + b) * L, n0, out);
     }
-    __syncthreads();      // the next row's prologue overwrites what the epilogue has just read
+    row_sync<P>();      // the next row's prologue overwrites what the epilogue has just read
   }
 }
 
@@ -249,11 +254,11 @@ __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
         dst[2 * q + 1] = make_float4(a.z, bq.z, a.w, bq.w);
       });
     }
-    __syncthreads();
+    row_sync<P>();
     cf x[16];
     fwd_load<P, P::R1, P::S1>(x, t, row);
     forward_to_pairs<P, false>(x, t, row, tw, g, g2);
-    __syncthreads();      // LDS is reused by the next row
+    row_sync<P>();      // LDS is reused by the next row
 
     float4 K[8];
     auto split = [&](cf za, cf zb) -> float4 {
