@@ -264,7 +264,8 @@ def main():
                    "launch": "one captured HIP graph per forward" if args.hip_graph else "eager launches",
                    "eager_ms_per_step": eager_ms,
                    "ms_per_step_with_cached_filter_spectra": cached_ms},
-        "roofline": {"kernel": "mixer_split_kernel (short conv + gates + two FFT long convs + add)",
+        "roofline": {"kernel": ("mixer_real_kernel" if L == 32768 else "mixer_split_kernel" if L >= 2048
+                                else "mixer_core_kernel") + " (short conv + gates + two FFT long convs + add)",
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MIXER_CORE_TRAFFIC_BYTES_C3 if args.config == "c3" else None,
