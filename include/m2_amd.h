@@ -84,14 +84,16 @@ int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int 
  * sub-transforms per row for 32768). */
 int m2_fftconv_supported_seqlen(int L);
 
-/* Bytes of the opaque spectrum buffer for d channels and sequence length L (both filters). */
+/* Bytes of the opaque spectrum buffer for d channels and sequence length L (both filters): 16 d L, and 24 d L at
+ * L = 32768 (where each frequency pair also carries the odd-sample spectrum times its twiddle).  Always ask. */
 size_t m2_filter_spectrum_bytes(int d, int L);
 
 /* taps1, taps2: (d, 2L) fp32 bidirectional taps of filter_fn and filter_fn2 (taps2 may be NULL:
  * treated as zero).  D1, D2: (d) fp32 skip weights (`filter_fn.bias`, `filter_fn2.bias`; either
  * may be NULL = 0): the reference's "+ u * D" term (hyena_utils.py:35) equals adding D to tap 0,
  * which is done here.  spec: m2_filter_spectrum_bytes(d, L) bytes; receives
- * rfft(taps + D e0, 2L)/(2L) of both filters in the order m2_mixer_core_fwd reads them. */
+ * rfft(taps + D e0, 2L)/(2L) of both filters (at L = 32768: of their even and odd samples) in the order
+ * m2_mixer_core_fwd reads them. */
 int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
                            int d, int L, void* stream);
 
