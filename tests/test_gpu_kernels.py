@@ -102,7 +102,8 @@ def test_plain_fftconv_module_api(gpu):
     assert rel_err(y, ref)[0] < TOL_F32
 
 
-@pytest.mark.parametrize("M,d,I", [(256, 768, 3072), (200, 256, 512), (4096, 1536, 6144)])
+@pytest.mark.parametrize("M,d,I", [(256, 768, 3072), (200, 256, 512), (4096, 1536, 6144), (300, 512, 2048),
+                                   (300, 1024, 4096), (130, 256, 768), (1100, 768, 3072)])
 def test_blockdiag_glu_and_linear(gpu, M, d, I):
     """K3 vs oracle.blockdiag_* on bf16-rounded operands (fp64 reference)."""
     from m2_amd import ops
