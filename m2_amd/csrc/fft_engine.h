@@ -29,11 +29,6 @@ struct Plan {
   static constexpr int RL = (R3 > 1) ? R3 : R2;   // radix of the least significant digit of a group index
   static constexpr int WG = T < 256 ? 256 : T;    // threads per workgroup
   static constexpr int RPW = WG / T;              // rows per workgroup
-  // Pass-1 twiddles: kept in registers for the whole kernel when the register budget allows it
-  // (up to 512 threads per workgroup), else only the base roots are kept and the powers are rebuilt
-  // where they are used (a 1024-thread workgroup has 128 registers per thread, and 30 long-lived
-  // twiddle registers would be spilled to memory and re-read for every row).
-  static constexpr bool P1_REGS = WG < 1024;
   static constexpr int ROW_LDS = N + (N >> 4);    // padded complex slots per row
   static constexpr int TW_LDS = R2 * (N / R1 / R2) + (R3_ > 1 ? R3_ * (N / R1 / R2 / R3_) : 0);   // twiddle tables
   static constexpr int WG_LDS = (T < 256 ? 256 / T : 1) * ROW_LDS + TW_LDS;                         // float2 slots per workgroup
@@ -85,7 +80,7 @@ __device__ __forceinline__ void row_sync() {
 // pass: tables in LDS ([k][m], conflict-free for consecutive m), built once per workgroup.
 template <class P>
 struct Twiddles {
-  cf p1[16 / P::R1][P::P1_REGS ? P::R1 : 2];     // [butterfly][k], k = 1 .. R1-1 (k = 1 only without P1_REGS)
+  cf p1[16 / P::R1][P::R1];     // [butterfly][k], k = 1 .. R1-1: pass-1 twiddles, in registers for the whole kernel
   const float2* tab2;           // [R2][S2]
   const float2* tab3;           // [R3][S3]   (R3 > 1 only)
   static constexpr int TAB2 = P::R2 * P::S2;
@@ -101,8 +96,7 @@ __device__ __forceinline__ void twiddles_init(Twiddles<P>& tw, int t, float2* ta
     constexpr int i = decltype(ii)::value;
     const int q = t + P::T * i;
     const cf w = unit_root(q % P::S1, P::S1 * P::R1);
-    if constexpr (P::P1_REGS) powers<P::R1>(w, tw.p1[i]);
-    else tw.p1[i][1] = w;
+    powers<P::R1>(w, tw.p1[i]);
   });
   tw.tab2 = tables;
   tw.tab3 = tables + Twiddles<P>::TAB2;
@@ -124,14 +118,7 @@ __device__ __forceinline__ void twiddles_init(Twiddles<P>& tw, int t, float2* ta
 // pass-1 twiddles pw[k] = w^k of butterfly I of this thread
 template <class P, int I>
 __device__ __forceinline__ void pass1_twiddles(const Twiddles<P>& tw, cf (&pw)[P::R1]) {
-  if constexpr (P::P1_REGS) {
-    static_for<1, P::R1>([&](auto k) { pw[decltype(k)::value] = tw.p1[I][decltype(k)::value]; });
-  } else {
-    cf w = tw.p1[I][1];
-    // opaque to the optimiser, so that the powers are rebuilt here and not hoisted out of the row loop
-    asm volatile("" : "+v"(w.re), "+v"(w.im));
-    powers<P::R1>(w, pw);
-  }
+  static_for<1, P::R1>([&](auto k) { pw[decltype(k)::value] = tw.p1[I][decltype(k)::value]; });
 }
 
 // twiddle w^(m k) of pass PASS (2 or 3), shared table in LDS

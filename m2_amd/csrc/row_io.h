@@ -8,33 +8,7 @@
 
 namespace m2 {
 
-// 8 consecutive activations starting at element n0 (n0 % 8 == 0) plus the two before them, as fp32:
-// out[0], out[1] = in[n0-2], in[n0-1] (zero when n0 == 0), out[2..10) = in[n0 .. n0+8).
-// `add` is added to every element that exists (the two before n0 == 0 stay zero: that is the
-// convolution's zero padding, which sits outside the biased signal).
-__device__ __forceinline__ void load10(const float* p, int n0, float add, float (&o)[10]) {
-  const float4 a = *reinterpret_cast<const float4*>(p + n0);
-  const float4 b = *reinterpret_cast<const float4*>(p + n0 + 4);
-  o[0] = 0.f; o[1] = 0.f;
-  if (n0 > 0) {
-    const float2 h = *reinterpret_cast<const float2*>(p + n0 - 2);
-    o[0] = h.x + add; o[1] = h.y + add;
-  }
-  o[2] = a.x + add; o[3] = a.y + add; o[4] = a.z + add; o[5] = a.w + add;
-  o[6] = b.x + add; o[7] = b.y + add; o[8] = b.z + add; o[9] = b.w + add;
-}
-__device__ __forceinline__ void load10(const uint16_t* p, int n0, float add, float (&o)[10]) {
-  const uint4 a = *reinterpret_cast<const uint4*>(p + n0);
-  o[0] = 0.f; o[1] = 0.f;
-  if (n0 > 0) {
-    const uint32_t h = *reinterpret_cast<const uint32_t*>(p + n0 - 2);
-    o[0] = __uint_as_float(h << 16) + add; o[1] = __uint_as_float(h & 0xffff0000u) + add;
-  }
-  o[2] = __uint_as_float(a.x << 16) + add; o[3] = __uint_as_float(a.x & 0xffff0000u) + add;
-  o[4] = __uint_as_float(a.y << 16) + add; o[5] = __uint_as_float(a.y & 0xffff0000u) + add;
-  o[6] = __uint_as_float(a.z << 16) + add; o[7] = __uint_as_float(a.z & 0xffff0000u) + add;
-  o[8] = __uint_as_float(a.w << 16) + add; o[9] = __uint_as_float(a.w & 0xffff0000u) + add;
-}
+// 8 consecutive outputs from fp32 registers, one or two 16-byte stores
 __device__ __forceinline__ void store8(float* p, int n0, const float (&v)[8]) {
   *reinterpret_cast<float4*>(p + n0) = make_float4(v[0], v[1], v[2], v[3]);
   *reinterpret_cast<float4*>(p + n0 + 4) = make_float4(v[4], v[5], v[6], v[7]);
@@ -48,8 +22,11 @@ __device__ __forceinline__ void store8(uint16_t* p, int n0, const float (&v)[8])
   *reinterpret_cast<uint4*>(p + n0) = o;
 }
 
-// The same accesses split into the loads (`fetch10`, raw bits) and the conversion (`expand10`), so that
-// a kernel can put all loads of a row in flight before it starts converting.
+// 8 consecutive activations starting at element n0 (n0 % 8 == 0) plus the two before them, as fp32:
+// out[0], out[1] = in[n0-2], in[n0-1] (zero when n0 == 0), out[2..10) = in[n0 .. n0+8); `add` is added to every
+// element that exists (the two before n0 == 0 stay zero: that is the convolution's zero padding, which sits
+// outside the biased signal).  Split into the loads (`fetch`, raw bits) and the conversion (`expand`), so that a
+// kernel can put all loads of a row in flight before it starts converting.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
