@@ -270,21 +270,17 @@ static int launch_blockdiag(const void* x, const void* w, const float* bias, con
 // barrier per chunk, the chunk after next in flight in registers); per K step of 16 a wave reads 2 A and 3 B
 // operands for 6 MFMAs.  Epilogue: bias + bf16 residual, rows leave through LDS 64 at a time as full segments.
 // ---------------------------------------------------------------------------------------------
-constexpr int kWideBN = 192;
-// WRG = row groups of 64: 4 (256 rows, 8 waves, one workgroup per compute unit, double-buffered LDS and two chunks
-// in flight in registers) or 2 (128 rows, 4 waves, one LDS stage, so that two workgroups share a compute unit and
-// one's epilogue overlaps the other's main loop).
-template <typename OUT, int WRG>
-__global__ __launch_bounds__(128 * WRG) __attribute__((amdgpu_waves_per_eu(2, 2))) void blockdiag_wide_kernel(
+constexpr int kWideBM = 256, kWideBN = 192;
+template <typename OUT>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void blockdiag_wide_kernel(
     const uint16_t* __restrict__ x,      // (M, nb p) bf16
     const uint16_t* __restrict__ w,      // (nb, q, p) bf16
     const float* __restrict__ bias,      // (nb q) or null
     const uint16_t* __restrict__ resid,  // (M, nb q) bf16 or null
     OUT* __restrict__ out,               // (M, nb q)
     int M, int nb, int p, int q) {
-  constexpr int BM = 64 * WRG, BN = kWideBN, NT = 128 * WRG;
-  constexpr bool TWO_STAGE = WRG == 4;
-  constexpr int A_CH = BM * (kBK / 8) / NT, B_CH = BN * (kBK / 8) / NT;        // chunks of 16 bytes per thread: 4 and 3 or 6
+  constexpr int BM = kWideBM, BN = kWideBN, NT = 512, WRG = BM / 64;
+  constexpr int A_CH = BM * (kBK / 8) / NT, B_CH = BN * (kBK / 8) / NT;        // chunks of 16 bytes per thread: 4 and 3
   constexpr int STAGE = (BM + BN) * kLdsRow;
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
@@ -321,7 +317,7 @@ __global__ __launch_bounds__(128 * WRG) __attribute__((amdgpu_waves_per_eu(2, 2)
   });
   // two chunks in flight in registers (ring slot = chunk & 1) on top of the one waiting in the other LDS stage:
   // with one workgroup per compute unit the loads in flight are what hides the memory latency
-  u32x4 ra[TWO_STAGE ? 2 : 1][A_CH], rb[TWO_STAGE ? 2 : 1][B_CH];
+  u32x4 ra[2][A_CH], rb[2][B_CH];
   auto gload = [&](int c, auto slot_) __attribute__((always_inline)) {
     constexpr int sl = decltype(slot_)::value;
     static_for<0, A_CH>([&](auto jj_) { ra[sl][decltype(jj_)::value] = *reinterpret_cast<const u32x4*>(pa[decltype(jj_)::value] + c * kBK); });
@@ -353,52 +349,35 @@ __global__ __launch_bounds__(128 * WRG) __attribute__((amdgpu_waves_per_eu(2, 2)
       });
     });
   };
-  if constexpr (TWO_STAGE) {
-    // chunk c is multiplied from LDS stage c & 1 while chunk c + 1 moves from ring slot (c + 1) & 1 to the other
-    // stage and chunk c + 3 is requested into that slot
-    auto step = [&](int c, auto par_) __attribute__((always_inline)) {
-      constexpr int nx = (decltype(par_)::value + 1) & 1;          // (c + 1) & 1
-      compute(c & 1);
-      if (c + 1 < nchunks) {
-        sstore(nx, ic<nx>{});                // that stage was last read before the barrier that ended chunk c - 1
-        if (c + 3 < nchunks) gload(c + 3, ic<nx>{});
-      }
-      __syncthreads();
-    };
-    gload(0, ic<0>{});
-    sstore(0, ic<0>{});
-    if (nchunks > 1) gload(1, ic<1>{});
-    if (nchunks > 2) gload(2, ic<0>{});
-    __syncthreads();
-    int c = 0;
-    for (; c + 1 < nchunks; c += 2) {
-      step(c, ic<0>{});
-      step(c + 1, ic<1>{});
+  // chunk c is multiplied from LDS stage c & 1 while chunk c + 1 moves from ring slot (c + 1) & 1 to the other
+  // stage and chunk c + 3 is requested into that slot
+  auto step = [&](int c, auto par_) __attribute__((always_inline)) {
+    constexpr int nx = (decltype(par_)::value + 1) & 1;          // (c + 1) & 1
+    compute(c & 1);
+    if (c + 1 < nchunks) {
+      sstore(nx, ic<nx>{});                // that stage was last read before the barrier that ended chunk c - 1
+      if (c + 3 < nchunks) gload(c + 3, ic<nx>{});
     }
-    if (c < nchunks) step(c, ic<0>{});
-  } else {
-    // one LDS stage: the next chunk waits in registers while this one is multiplied (two barriers per chunk)
-    gload(0, ic<0>{});
-    sstore(0, ic<0>{});
-    if (nchunks > 1) gload(1, ic<0>{});
     __syncthreads();
-    for (int c = 0; c < nchunks; ++c) {
-      compute(0);
-      __syncthreads();
-      if (c + 1 < nchunks) {
-        sstore(0, ic<0>{});
-        if (c + 2 < nchunks) gload(c + 2, ic<0>{});
-      }
-      __syncthreads();
-    }
+  };
+  gload(0, ic<0>{});
+  sstore(0, ic<0>{});
+  if (nchunks > 1) gload(1, ic<1>{});
+  if (nchunks > 2) gload(2, ic<0>{});
+  __syncthreads();
+  int c = 0;
+  for (; c + 1 < nchunks; c += 2) {
+    step(c, ic<0>{});
+    step(c + 1, ic<1>{});
   }
+  if (c < nchunks) step(c, ic<0>{});
 
   // ---- epilogue: 64 rows at a time (the rows of wave row group ep) through an fp32 LDS tile.  The residual
   // values of a pass are requested one pass ahead, all at once: loaded where they are used, every row of the
   // copy loop waited a full memory latency ----
   constexpr int OROW = BN + 4;
-  constexpr int TPR = BN / 4, RPI = NT / TPR;           // 48 threads per row: 10 or 5 rows per sweep
-  constexpr int NR = (64 + RPI - 1) / RPI;              // rows per thread and pass: 7 or 13
+  constexpr int TPR = BN / 4, RPI = NT / TPR;           // 48 threads per row, 10 rows per sweep (32 threads idle)
+  constexpr int NR = (64 + RPI - 1) / RPI;              // rows per thread and pass: 7
   float* so_base = reinterpret_cast<float*>(smem);
   const int cq = (tid % TPR) * 4, r0 = tid / TPR;
   float4 bq = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -456,20 +435,12 @@ __global__ __launch_bounds__(128 * WRG) __attribute__((amdgpu_waves_per_eu(2, 2)
 template <typename OUT>
 static int launch_blockdiag_wide(const void* x, const void* w, const float* bias, const void* resid, void* out, int M,
                                  int nb, int p, int q, hipStream_t stream) {
-  // 128-row tiles (two workgroups per compute unit) once there are enough of them to fill the chip twice over
-  const bool small = (long)((M + 127) / 128) * (nb * q / kWideBN) >= 4L * num_cus();
-  const int bm = small ? 128 : 256;
-  const size_t stage = (size_t)(bm + kWideBN) * kLdsRow * sizeof(uint16_t);
-  const size_t epi = (size_t)64 * (kWideBN + 4) * sizeof(float);
-  size_t lds = small ? stage : 2 * stage;
-  if (lds < epi) lds = epi;
-  auto kern = small ? blockdiag_wide_kernel<OUT, 2> : blockdiag_wide_kernel<OUT, 4>;
-  if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(blockdiag_wide): %s", hipGetErrorString(e));
-  }
-  dim3 grid(((M + bm - 1) / bm) * (nb * q / kWideBN));
-  hipLaunchKernelGGL(kern, grid, dim3(2 * bm), lds, stream, (const uint16_t*)x, (const uint16_t*)w, bias,
+  const size_t lds = (size_t)2 * (kWideBM + kWideBN) * kLdsRow * sizeof(uint16_t);      // 129 KB; the epilogue tile (50 KB) reuses it
+  auto kern = blockdiag_wide_kernel<OUT>;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(blockdiag_wide): %s", hipGetErrorString(e));
+  dim3 grid(((M + kWideBM - 1) / kWideBM) * (nb * q / kWideBN));
+  hipLaunchKernelGGL(kern, grid, dim3(512), lds, stream, (const uint16_t*)x, (const uint16_t*)w, bias,
                      (const uint16_t*)resid, (OUT*)out, M, nb, p, q);
   return check_launch("blockdiag_wide");
 }
@@ -888,9 +859,17 @@ static int launch_glu_ws(const void* x, const void* w, void* out, int M, int nb,
     if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(blockdiag_glu_ws): %s", hipGetErrorString(e));
   }
   const int nslices = I / ncols;
-  // rows per workgroup: long runs amortise the weight load, but keep at least ~3 workgroups per CU
+  // Rows per workgroup (a multiple of the 32-row slab): long runs amortise the weight load and the first slab's
+  // latency (worth about three slab steps), but the workgroups should fill the chip in whole rounds.  Cost model:
+  // rounds x (3 + slabs per workgroup), minimised over the candidates.
+  const long slots = (long)num_cus() * (wide || !PIPELINED ? 1 : 2);
   int rows = 512;
-  while (rows > 128 && (long)nslices * ((M + rows - 1) / rows) < 3L * num_cus()) rows >>= 1;
+  long best = -1;
+  for (int cand = 64; cand <= 1024; cand += 32) {
+    const long wgs = (long)nslices * ((M + cand - 1) / cand);
+    const long cost = ((wgs + slots - 1) / slots) * (3 + cand / 32);
+    if (best < 0 || cost < best) { best = cost; rows = cand; }
+  }
   const int nchunks = (M + rows - 1) / rows;
   hipLaunchKernelGGL(kern, dim3(nslices * nchunks), dim3(wide ? 64 * NW : 256), lds, stream, (const uint16_t*)x,
                      (const uint16_t*)w, (uint16_t*)out, M, nb, q, rows);
@@ -946,7 +925,9 @@ extern "C" int m2_blockdiag_linear_fwd(const void* x, const void* w, const float
   int rc = check_blockdiag("m2_blockdiag_linear_fwd", M, nblocks, p, q, false);
   if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
-  if (q % kWideBN == 0)
+  // 256 x 192 tiles once there is at least one per compute unit (measured at d = 768 and 1536: below that the
+  // smaller tiles of the general kernel fill the chip better)
+  if (q % kWideBN == 0 && (long)((M + kWideBM - 1) / kWideBM) * (nblocks * q / kWideBN) >= num_cus())
     return out_dtype == M2_DTYPE_F32 ? launch_blockdiag_wide<float>(x, w, bias, residual, out, M, nblocks, p, q, st)
                                      : launch_blockdiag_wide<uint16_t>(x, w, bias, residual, out, M, nblocks, p, q, st);
   const bool wide = q % 128 == 0;
