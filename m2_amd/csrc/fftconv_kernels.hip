@@ -304,9 +304,21 @@ static int launch_mixer_core(const void* xproj, const float* u, const float* sw,
   }
   const int rows_per_xcd = (d / 8) * B;
   const int slots_needed = (rows_per_xcd + P::RPW - 1) / P::RPW;
-  const int per_cu = (int)((160 * 1024) / lds_bytes) < 1 ? 1 : (int)((160 * 1024) / lds_bytes);
+  // workgroups that are resident on a compute unit at once (registers or LDS, whichever binds): asked once per
+  // kernel, the LDS bound is the fallback
+  static int resident = 0;
+  if (resident == 0) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)kern, P::WG, lds_bytes) != hipSuccess || n < 1)
+      n = (int)((160 * 1024) / lds_bytes) < 1 ? 1 : (int)((160 * 1024) / lds_bytes);
+    resident = n;
+  }
+  const int per_cu = resident;
   int slots = (num_cus() / 8) * (per_cu > 8 ? 8 : per_cu);          // workgroups per XCD
   if (slots > slots_needed) slots = slots_needed;
+  // every workgroup the same number of row batches: the fewest workgroups that need no extra round
+  const int rounds = (slots_needed + slots - 1) / slots;
+  slots = (slots_needed + rounds - 1) / rounds;
   const int grid = 8 * slots;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(P::WG), lds_bytes, stream, (const ACT*)xproj, u, sw, sb, pbias,
                      (const float4*)spec, (ACT*)y, B, d);

@@ -455,6 +455,8 @@ static int launch_mixer_real(const void* xproj, const float* u, const float* sw,
   const int rows_per_xcd = (d / 8) * B;
   int slots = num_cus() / 8;          // one workgroup per compute unit (140 KB of LDS)
   if (slots > rows_per_xcd) slots = rows_per_xcd;
+  const int rounds = (rows_per_xcd + slots - 1) / slots;      // every workgroup the same number of rows
+  slots = (rows_per_xcd + rounds - 1) / rounds;
   hipLaunchKernelGGL(kern, dim3(8 * slots), dim3(P::T), lds_bytes, stream, (const ACT*)xproj, u, sw, sb, pbias, spec,
                      (ACT*)y, B, d);
   return check_launch("mixer_real");

@@ -309,6 +309,8 @@ static int launch_mixer_split(const void* xproj, const float* u, const float* sw
   if (per_cu > 512 / P::T) per_cu = 512 / P::T;  // two waves per SIMD at 256 registers
   int slots = (num_cus() / 8) * per_cu;          // workgroups per XCD
   if (slots > rows_per_xcd) slots = rows_per_xcd;
+  const int rounds = (rows_per_xcd + slots - 1) / slots;      // every workgroup the same number of rows
+  slots = (rows_per_xcd + rounds - 1) / rounds;
   hipLaunchKernelGGL(kern, dim3(8 * slots), dim3(P::T), lds_bytes, stream, (const ACT*)xproj, u, sw, sb, pbias,
                      (const float4*)spec, (ACT*)y, B, d);
   return check_launch("mixer_split");
