@@ -865,7 +865,7 @@ static int launch_glu_ws(const void* x, const void* w, void* out, int M, int nb,
   const long slots = (long)num_cus() * (wide || !PIPELINED ? 1 : 2);
   int rows = 512;
   long best = -1;
-  for (int cand = 64; cand <= 1024; cand += 32) {
+  for (int cand = 64; cand <= 4096; cand += 32) {
     const long wgs = (long)nslices * ((M + cand - 1) / cand);
     const long cost = ((wgs + slots - 1) / slots) * (3 + cand / 32);
     if (best < 0 || cost < best) { best = cost; rows = cand; }
