@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM-side bytes per mixer-core launch at the default workload, from the two rocprofv3 --pmc runs
 # (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000 against a plain 256 MiB copy); summary in
 # profiles/mixer_core_L8192_B4_hbm_traffic.md.  Only valid for --config c3.
-MIXER_CORE_TRAFFIC_BYTES_C3 = int((193770 * 2.0 + 67419 * 1.0) * 1024)
+MIXER_CORE_TRAFFIC_BYTES_C3 = int((194033 * 2.0 + 67345 * 1.0) * 1024)
 
 
 def workload(name: str):
