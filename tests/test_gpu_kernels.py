@@ -501,10 +501,11 @@ def test_mixer_variants_without_reverse_filter_or_residual_conv(gpu, L, bidirect
 
 
 def test_plain_fftconv_long_rows(gpu):
-    """m2_fftconv_fwd (one filter, no short conv, no gates) on the split kernels, fp32 and bf16 storage."""
+    """m2_fftconv_fwd (one filter, no short conv, no gates) on the half-transform kernels (L = 2048 .. 16384) and the
+    real-signal kernel (L = 32768), fp32 and bf16 storage."""
     from m2_amd import ops
     from oracle import m2_oracle as O
-    for L in (4096, 8192):
+    for L in (2048, 4096, 8192, 16384, 32768):
         d, B = 16, 2
         g = torch.Generator().manual_seed(L)
         x = torch.randn(d, B, L, generator=g)
