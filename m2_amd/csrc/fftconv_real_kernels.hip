@@ -331,7 +331,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
 }
 
 // ------------------------------------------------------------------------------------------
-// filter taps -> (Ke, Ko, w Ko) in the layout above; work item = (channel, filter, half transform)
+// filter taps -> (Ke, Ko, w Ko) in the layout above; work item = (channel, filter), both half transforms
 // ------------------------------------------------------------------------------------------
 template <class P>
 __global__ __launch_bounds__(P::T) void filter_spectrum_real_kernel(
@@ -355,39 +355,55 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_real_kernel(
   const float scale = 0.25f / (float)H;
   __syncthreads();
 
-  for (int item = blockIdx.x; item < 4 * d; item += gridDim.x) {
-    const int c = item >> 2, f = (item >> 1) & 1;
+  // work item = (channel, filter): the taps row is read once; its even-half combination goes to LDS at once, the
+  // odd-half combination waits in registers (64) while the even half is transformed
+  for (int item = blockIdx.x; item < 2 * d; item += gridDim.x) {
+    const int c = item >> 1, f = item & 1;
     const float* taps = f ? taps2 : taps1;
     const float* D = f ? D2 : D1;
-    float4* sp4 = reinterpret_cast<float4*>(spec + (long)item * BLK) + t;
-    float2* sp2 = reinterpret_cast<float2*>(spec + (long)item * BLK + 64L * T) + t;
+    float* blk = spec + (long)item * 2 * BLK;
     if (!taps) {
-      static_for<0, 16>([&](auto ss) {
-        constexpr int s = decltype(ss)::value;
-        sp4[s * T] = make_float4(0.f, 0.f, 0.f, 0.f);
-        sp2[s * T] = make_float2(0.f, 0.f);
+      static_for<0, 2>([&](auto hh) {
+        float4* z4 = reinterpret_cast<float4*>(blk + decltype(hh)::value * BLK) + t;
+        float2* z2 = reinterpret_cast<float2*>(blk + decltype(hh)::value * BLK + 64L * T) + t;
+        static_for<0, 16>([&](auto ss) {
+          constexpr int s = decltype(ss)::value;
+          z4[s * T] = make_float4(0.f, 0.f, 0.f, 0.f);
+          z2[s * T] = make_float2(0.f, 0.f);
+        });
       });
       continue;
     }
+    // g[m] = taps[2m] + i taps[2m+1], m < H; even half: g_lo + g_hi, odd half: g_lo - g_hi
+    constexpr int Q = NS / 2 / T;
+    f32x4_t od[Q];
+    {
+      f32x4_t lo[Q], hi[Q];
+      static_for<0, Q>([&](auto qq) {
+        constexpr int q = decltype(qq)::value;
+        const float* p = taps + (long)c * 2 * H + 4 * (q * T + t);
+        lo[q] = *reinterpret_cast<const f32x4_t*>(p);
+        hi[q] = *reinterpret_cast<const f32x4_t*>(p + 2 * NS);
+      });
+      if (D && t == 0) lo[0].x += D[c];      // the skip weight is one more tap at lag 0
+      static_for<0, Q>([&](auto qq) {
+        constexpr int q = decltype(qq)::value;
+        float2* dst = row + sphys(2 * (q * T + t));     // 2 consecutive slots never straddle a pad
+        dst[0] = make_float2(lo[q].x + hi[q].x, lo[q].y + hi[q].y);
+        dst[1] = make_float2(lo[q].z + hi[q].z, lo[q].w + hi[q].w);
+        od[q] = lo[q] - hi[q];
+      });
+    }
     auto one_half = [&](auto hh) __attribute__((always_inline)) {
       constexpr bool ODD = decltype(hh)::value == 1;
-      // g[m] = taps[2m] + i taps[2m+1], m < H; even half: g_lo + g_hi, odd half: g_lo - g_hi
-      {
-        constexpr int Q = NS / 2 / T;
-        f32x4_t lo[Q], hi[Q];
+      float4* sp4 = reinterpret_cast<float4*>(blk + (ODD ? BLK : 0)) + t;
+      float2* sp2 = reinterpret_cast<float2*>(blk + (ODD ? BLK : 0) + 64L * T) + t;
+      if constexpr (ODD) {
         static_for<0, Q>([&](auto qq) {
           constexpr int q = decltype(qq)::value;
-          const float* p = taps + (long)c * 2 * H + 4 * (q * T + t);
-          lo[q] = *reinterpret_cast<const f32x4_t*>(p);
-          hi[q] = *reinterpret_cast<const f32x4_t*>(p + 2 * NS);
-        });
-        if (D && t == 0) lo[0].x += D[c];      // the skip weight is one more tap at lag 0
-        constexpr float sgn = ODD ? -1.f : 1.f;
-        static_for<0, Q>([&](auto qq) {
-          constexpr int q = decltype(qq)::value;
-          float2* dst = row + sphys(2 * (q * T + t));     // 2 consecutive slots never straddle a pad
-          dst[0] = make_float2(lo[q].x + sgn * hi[q].x, lo[q].y + sgn * hi[q].y);
-          dst[1] = make_float2(lo[q].z + sgn * hi[q].z, lo[q].w + sgn * hi[q].w);
+          float2* dst = row + sphys(2 * (q * T + t));
+          dst[0] = make_float2(od[q].x, od[q].y);
+          dst[1] = make_float2(od[q].z, od[q].w);
         });
       }
       __syncthreads();
@@ -399,39 +415,44 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_real_kernel(
       __syncthreads();
       const int ga = ODD ? grp.go : grp.ge, gb = ODD ? grp.gc : grp.gm;
       fwd_groups<P>(x, row, ga, gb);
-      __syncthreads();      // LDS is restaged by the next item
+      __syncthreads();      // LDS is restaged by the next half / item
 
       // (Ke, Ko) of the pair (za at frequency k of this half transform, zb at its partner), and w_H^kk Ko with
-      // kk = 2 k + ODD the frequency of za in the H-point transform
-      auto emit = [&](int s, cf za, cf zb, int k) __attribute__((always_inline)) {
+      // kk = 2 k + ODD the frequency of za in the H-point transform.  k = k0 + R1 R2 s for slot s of a group,
+      // so the root is w_H^(2 k0 + ODD) (one sincos per group) times the constant w_16^s.
+      auto emit = [&](auto ss, auto slot, cf za, cf zb, cf beta) __attribute__((always_inline)) {
+        constexpr int s = decltype(ss)::value;
         const cf ke = {scale * (za.re + zb.re), scale * (za.im - zb.im)};
         const cf ko = {scale * (za.im + zb.im), scale * (zb.re - za.re)};
-        const cf kw = cmul(unit_root(2 * k + (ODD ? 1 : 0), H), ko);
-        sp4[s * T] = make_float4(ke.re, ke.im, ko.re, ko.im);
-        sp2[s * T] = make_float2(kw.re, kw.im);
+        const cf kw = cmul(beta, mul_w64<4 * s, false>(ko));
+        sp4[decltype(slot)::value * T] = make_float4(ke.re, ke.im, ko.re, ko.im);
+        sp2[decltype(slot)::value * T] = make_float2(kw.re, kw.im);
       };
-      const int kbase = ga / R2 + R1 * (ga % R2);       // frequency of slot 0 of group ga
       if (!ODD && grp.special) {
         const cf z0 = x[bitrev(0, 4)], zn = x[bitrev(8, 4)];
         sp4[0] = make_float4(4.f * scale * z0.re, 4.f * scale * z0.im, 4.f * scale * zn.re, 4.f * scale * zn.im);
         sp2[0] = make_float2(0.f, 0.f);
+        const cf one = {1.f, 0.f};                                  // group 0: k0 = 0
         static_for<1, 8>([&](auto ss) {
           constexpr int s = decltype(ss)::value;
-          emit(s, x[bitrev(s, 4)], x[bitrev(16 - s, 4)], R1 * R2 * s);
+          emit(ss, ss, x[bitrev(s, 4)], x[bitrev(16 - s, 4)], one);
         });
+        const cf beta = unit_root(2 * (R1 * (R2 / 2)), H);          // group R2/2: k0 = R1 R2 / 2
         static_for<0, 8>([&](auto ss) {
           constexpr int s = decltype(ss)::value;
-          emit(8 + s, x[16 + bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], R1 * (R2 / 2) + R1 * R2 * s);
+          emit(ss, ic<8 + s>{}, x[16 + bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], beta);
         });
       } else {
+        const int k0 = ga / R2 + R1 * (ga % R2);                    // frequency of slot 0 of group ga
+        const cf beta = unit_root(2 * k0 + (ODD ? 1 : 0), H);
         static_for<0, 16>([&](auto ss) {
           constexpr int s = decltype(ss)::value;
-          emit(s, x[bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], kbase + R1 * R2 * s);
+          emit(ss, ss, x[bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], beta);
         });
       }
     };
-    if (item & 1) one_half(ic<1>{});
-    else one_half(ic<0>{});
+    one_half(ic<0>{});
+    one_half(ic<1>{});
   }
 }
 
@@ -476,7 +497,7 @@ int launch_filter_spectrum_real(const float* taps1, const float* taps2, const fl
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(filter_spectrum_real): %s", hipGetErrorString(e));
   int grid = num_cus();
-  if (grid > 4 * d) grid = 4 * d;
+  if (grid > 2 * d) grid = 2 * d;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(P::T), lds_bytes, stream, taps1, taps2, D1, D2, spec, d);
   return check_launch("filter_spectrum_real");
 }
