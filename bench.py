@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Throughput of the M2-BERT-80M encoder forward on one MI355X, sequences per second.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c2|c4|c5] [--no-cpu-baseline] [--eager]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--reps R] [--config c3|c2|c4|c5|l512|l1024|l2048|l4096]
+                    [--no-cpu-baseline] [--eager]
 
 A step is one forward of embeddings + 12 Monarch-Mixer layers over one synthetic batch that is
 already resident in HBM (token ids on the GPU; filters are regenerated from the weights in every
@@ -10,12 +11,25 @@ L = 8192, batch 4 (BASELINE config index 2).  One JSON line is printed:
 
   value / ms_per_step   whole forward, wall clock bracketed by torch.cuda.synchronize(); the K timed steps
                         replay the forward (filter generation included) as one captured HIP graph
-                        (--eager: plain launches); config.eager_ms_per_step is the same K steps launched
-                        eagerly with the per-launch events below in between
-  roofline              the fused mixer-core kernel: algorithmic bytes per launch divided by its average
-                        duration, measured with HIP events around every launch of the K eager steps
+                        (--eager: plain launches).  The K steps are timed R times back to back (--reps,
+                        default 5): value is the median repetition, `repetitions` holds min / median / max.
+                        config.eager_ms_per_step is the same K steps launched eagerly with the per-launch
+                        events below in between
+  roofline              the fused mixer-core kernel against the HBM roof: algorithmic bytes per launch divided
+                        by its average duration PLUS the duration of the separate filter-generation kernels of
+                        the same layer (their output is what the formula credits as "filters read once");
+                        the core kernel on its own is reported beside it (`core_only_*`).  Durations from HIP
+                        events around every launch of the K eager steps
+  roofline_k3           the block-diagonal GEMMs against the bf16 MFMA roof, same event timing
   cpu_baseline          the CPU oracle (plain PyTorch fp32 restatement of the reference path) timed on
-                        this host's cores on the same inputs and weights
+                        this host's cores on the same inputs and weights: one warm-up forward, three timed,
+                        the median reported
+  parity_vs_cpu_oracle  every layer of the GPU forward against the fp32 oracle run on the GPU's own
+                        previous-layer output; the process exits with status 1 when a layer exceeds 2e-2
+
+The configs l512 .. l4096 are the reference's own benchmark grid (bert/README.md:154-162,
+bert/benchmark_fwd.py:62-80: (L, B) = (512, 32), (1024, 32), (2048, 16), (4096, 8), with c3 = (8192, 4));
+for those `tokens_per_ms`, the unit the reference prints, is reported beside seq/s.
 
 Only one GPU is used; --gpus N with N > 1 exits with a message.
 """
@@ -30,10 +44,14 @@ import time
 import torch
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM-side bytes per mixer-core launch at the default workload, from the two rocprofv3 --pmc runs
 # (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000 against a plain 256 MiB copy); summary in
 # profiles/mixer_core_L8192_B4_hbm_traffic.md.  Only valid for --config c3.
 MIXER_CORE_TRAFFIC_BYTES_C3 = int((194033 * 2.0 + 67345 * 1.0) * 1024)
+
+
+REFERENCE_GRID = {"l512": (512, 32), "l1024": (1024, 32), "l2048": (2048, 16), "l4096": (4096, 8)}
 
 
 def workload(name: str):
@@ -54,6 +72,11 @@ def workload(name: str):
         cfg, B, pad = m2_amd.m2_bert_large(128, 24), 64, False
         label = "M2-BERT large 24x1536 encoder fwd, L=128, B=64 (config 4)"
         idx = 4
+    elif name in REFERENCE_GRID:
+        Lg, B = REFERENCE_GRID[name]
+        cfg, pad = m2_amd.m2_bert_80m(Lg), False
+        label = f"M2-BERT-80M encoder fwd, L={Lg}, B={B} (the reference's benchmark grid)"
+        idx = 10 + list(REFERENCE_GRID).index(name)
     else:
         raise SystemExit(f"unknown config {name}")
     gen = torch.Generator().manual_seed(1234 + idx)
@@ -108,19 +131,25 @@ class KernelTimer:
 
 
 def cpu_baseline(sd, cfg, ids, mask, B):
+    """The oracle's forward on this host: one warm-up forward, three timed, the median."""
     from oracle import m2_oracle as O
     # the thread count the box grants (OMP_NUM_THREADS is set there), not every core the host shows
-    cores = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(cores)
+    granted = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(granted)
+    times = []
     with torch.no_grad():
-        x = O.embeddings_forward(sd, "embeddings.", ids, cfg)
-        O.layer_forward(sd, "encoder.layer.0.", x, cfg)            # warm-up: one layer
-        t0 = time.perf_counter()
-        ref = O.model_forward(sd, ids, mask, cfg)
-        dt = time.perf_counter() - t0
+        ref = O.model_forward(sd, ids, mask, cfg)                   # warm-up (and the parity reference)
+        for _ in range(3):
+            t0 = time.perf_counter()
+            O.model_forward(sd, ids, mask, cfg)
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    dt = times[1]
     return ref, {"value": B / dt, "unit": "seq/s", "cores": torch.get_num_threads(), "kind": "port",
-                 "sample": f"one full forward (embeddings + {cfg.num_hidden_layers} layers) of the same batch, "
-                           f"fp32 torch.fft/einsum oracle, {dt:.2f} s after a one-layer warm-up"}
+                 "host_cpu_count": os.cpu_count(),
+                 "sample": f"full forward (embeddings + {cfg.num_hidden_layers} layers) of the same batch, fp32 "
+                           f"torch.fft/einsum oracle: 1 warm-up + 3 timed, median {dt:.2f} s "
+                           f"(min {times[0]:.2f}, max {times[2]:.2f})"}
 
 
 def main():
@@ -128,6 +157,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--reps", type=int, default=5, help="how many times the K timed steps are repeated (median reported)")
     ap.add_argument("--config", default="c3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", dest="hip_graph", action="store_false",
@@ -170,6 +200,7 @@ def main():
     model.load_state_dict(sd)
     model = model.to(dev).eval()
     ids_g, mask_g = ids.to(dev), mask.to(dev)
+    model.validate_ids = False          # the out-of-range flag is read once after the timed region, not every step
 
     timer = KernelTimer()
     wrapped = {}
@@ -196,17 +227,24 @@ def main():
     n_core = timer.count("mixer_core")
     for fn, orig in wrapped.items():            # per-launch events are only wanted for the eager timed steps
         setattr(ops, fn, orig)
+
+    def timed_steps():
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            model(ids_g, attention_mask=mask_g)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
     if args.hip_graph:
         model.encoder.use_hip_graph = True
-        with torch.no_grad():
-            for _ in range(max(2, args.warmup)):
-                out, _ = model(ids_g, attention_mask=mask_g)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(args.steps):
-                out, _ = model(ids_g, attention_mask=mask_g)
-            torch.cuda.synchronize()
-            dt = time.perf_counter() - t0
+    with torch.no_grad():
+        for _ in range(max(2, args.warmup)):
+            out, _ = model(ids_g, attention_mask=mask_g)
+        torch.cuda.synchronize()
+        reps = sorted(timed_steps() for _ in range(max(1, args.reps)))
+        out, _ = model(ids_g, attention_mask=mask_g)
+    model.embeddings.check_indices()
+    dt = reps[len(reps) // 2]
     ms = dt / args.steps * 1e3
     value = B / (dt / args.steps)
 
@@ -231,27 +269,34 @@ def main():
     t_core = means["mixer_core"]
     t_filt = means["filter_taps"] + means["filter_spectrum"]
     nbytes = mixer_core_bytes(B, L, d, 2)
-    achieved = nbytes / (t_core * 1e-3) / 1e9
+    core_only = nbytes / (t_core * 1e-3) / 1e9
+    achieved = nbytes / ((t_core + t_filt) * 1e-3) / 1e9
     I = cfg.intermediate_size
     M = B * L
-    glu_flops = 2 * M * d * 2 * I / cfg.monarch_mlp_nblocks
-    wo_flops = 2 * M * I * d / cfg.monarch_mlp_nblocks
+    nbk = cfg.monarch_mlp_nblocks
+    glu_flops = 2 * M * d * 2 * I / nbk
+    wo_flops = 2 * M * I * d / nbk
     t_glu = means["blockdiag_glu"]
-    mfma = {"glu_tflops": glu_flops / (t_glu * 1e-3) / 1e12, "peak_tflops": 2500.0,
-            "glu_frac": glu_flops / (t_glu * 1e-3) / 1e12 / 2500.0}
     # the same kernels against the HBM roof: algorithmic bytes (bf16 in, fused GLU write; wo with its bf16 residual
     # and fp32 sum) over the measured time, as a fraction of 8 TB/s
-    nbk = cfg.monarch_mlp_nblocks
     glu_bytes = M * d * 2 + (2 * I * d // nbk) * 2 + M * I * 2
     wo_bytes = M * I * 2 + (I * d // nbk) * 2 + M * d * 2 + M * d * 4
-    mfma["glu_hbm_frac"] = glu_bytes / (t_glu * 1e-3) / 1e9 / HBM_PEAK_GBPS
+    glu_tflops = glu_flops / (t_glu * 1e-3) / 1e12
+    k3 = {"kernel": "gated block-diagonal GEMM + GLU (m2_blockdiag_glu_fwd)", "bound": "mfma", "achieved": glu_tflops,
+          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": glu_tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+          "flops_per_launch": glu_flops, "ms_per_launch": t_glu,
+          "hbm_frac": glu_bytes / (t_glu * 1e-3) / 1e9 / HBM_PEAK_GBPS}
     if "wo_layernorm" in means:        # wo + bias + residual + LayerNorm as one kernel (an option, d <= 768)
-        mfma["wo_layernorm_tflops"] = wo_flops / (means["wo_layernorm"] * 1e-3) / 1e12
+        t_wo = means["wo_layernorm"]
+        k3["wo_kernel"] = "wo + bias + residual + LayerNorm (m2_blockdiag_linear_layernorm_fwd)"
     else:
         t_wo = means["blockdiag_linear"]
-        mfma["wo_tflops"] = wo_flops / (t_wo * 1e-3) / 1e12
-        mfma["wo_frac"] = mfma["wo_tflops"] / 2500.0
-        mfma["wo_hbm_frac"] = wo_bytes / (t_wo * 1e-3) / 1e9 / HBM_PEAK_GBPS
+        k3["wo_kernel"] = "wo + bias + residual (m2_blockdiag_linear_fwd)"
+        k3["wo_hbm_frac"] = wo_bytes / (t_wo * 1e-3) / 1e9 / HBM_PEAK_GBPS
+    k3["wo_achieved"] = wo_flops / (t_wo * 1e-3) / 1e12
+    k3["wo_frac"] = k3["wo_achieved"] / MFMA_BF16_PEAK_TFLOPS
+    k3["wo_ms_per_launch"] = t_wo
+    k3["both_frac"] = (glu_flops + wo_flops) / ((t_glu + t_wo) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
 
     result = {
         "metric": "seq/s M2-BERT-80M fwd at L=8192; FFT-conv HBM GB/s & % of peak" if args.config == "c3"
@@ -264,41 +309,56 @@ def main():
                    "launch": "one captured HIP graph per forward" if args.hip_graph else "eager launches",
                    "eager_ms_per_step": eager_ms,
                    "ms_per_step_with_cached_filter_spectra": cached_ms},
+        "repetitions": {"count": len(reps), "steps_each": args.steps, "ms_per_step_min": reps[0] / args.steps * 1e3,
+                        "ms_per_step_median": ms, "ms_per_step_max": reps[-1] / args.steps * 1e3,
+                        "timed_seconds_total": sum(reps)},
+        "tokens_per_ms": B * L / ms,
         "roofline": {"kernel": ("mixer_real_kernel" if L == 32768 else "mixer_split_kernel" if L >= 2048
-                                else "mixer_core_kernel") + " (short conv + gates + two FFT long convs + add)",
+                                else "mixer_core_kernel") + " (short conv + gates + two FFT long convs + add)"
+                               " with the filter-generation kernels of the layer",
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MIXER_CORE_TRAFFIC_BYTES_C3 if args.config == "c3" else None,
-                     "bytes_per_launch": nbytes, "ms_per_launch": t_core, "launches_timed": n_core,
-                     "achieved_incl_filter_generation": nbytes / ((t_core + t_filt) * 1e-3) / 1e9,
+                     "bytes_per_launch": nbytes, "ms_per_launch": t_core + t_filt, "launches_timed": n_core,
+                     "core_only_ms_per_launch": t_core, "core_only_achieved": core_only,
+                     "core_only_frac": core_only / HBM_PEAK_GBPS,
                      "filter_generation_ms_per_layer": t_filt},
+        "roofline_k3": k3,
         "kernels_ms_per_layer": means,
-        "blockdiag_mfma": mfma,
     }
+    failed = False
     if not args.no_cpu_baseline:
         ref, cb = cpu_baseline(sd, cfg, ids, mask, B)
         result["cpu_baseline"] = cb
         o = out.float().cpu().double()
         r = ref.double()
-        # the 2e-2 bar is per layer: the last layer of the GPU forward against the fp32 oracle run on the GPU's own
-        # previous-layer output.  End to end the network amplifies bf16 rounding with depth (the reference's own
-        # autocast rounding points, restated on the CPU, drift further from the fp32 oracle than this path does),
-        # so that figure is reported beside it, not held to the bar.
+        # The 2e-2 bar is held per layer, for every layer: layer i of the GPU forward against the fp32 oracle run on
+        # the GPU's own output of layer i - 1.  End to end a deep long-sequence stack amplifies bf16 rounding (at
+        # L = 8192 the reference's own autocast numerics drift from the fp32 path just as far; a GPU test measures
+        # that), so the end-to-end figure is reported beside it and held to the bar only where it stays inside it.
         from oracle import m2_oracle as O
         model.encoder.use_hip_graph = False
         with torch.no_grad():
             layers, _ = model(ids_g, attention_mask=mask_g, output_all_encoded_layers=True)
-            n = cfg.num_hidden_layers
-            prev = layers[n - 2].float().cpu() if n > 1 else O.embeddings_forward(sd, "embeddings.", ids, cfg)
-            want = O.layer_forward(sd, f"encoder.layer.{n - 1}.", prev, cfg).double()
-            got = layers[n - 1].float().cpu().double()
+            prev = O.embeddings_forward(sd, "embeddings.", ids, cfg)
+            per_layer = []
+            for i in range(cfg.num_hidden_layers):
+                want = O.layer_forward(sd, f"encoder.layer.{i}.", prev, cfg).double()
+                got = layers[i].float().cpu()
+                per_layer.append([((got.double() - want).abs().max() / want.abs().max()).item(),
+                                  ((got.double() - want).norm() / want.norm()).item()])
+                prev = got
+        worst = max(max(p) for p in per_layer)
         result["parity_vs_cpu_oracle"] = {
-            "per_layer_max_rel": ((got - want).abs().max() / want.abs().max()).item(),
-            "per_layer_l2_rel": ((got - want).norm() / want.norm()).item(), "tolerance": 2e-2,
-            "layer": n - 1,
+            "per_layer_max_rel": max(p[0] for p in per_layer), "per_layer_l2_rel": max(p[1] for p in per_layer),
+            "per_layer": per_layer, "tolerance": 2e-2, "layers_checked": cfg.num_hidden_layers,
             "end_to_end_max_rel": ((o - r).abs().max() / r.abs().max()).item(),
             "end_to_end_l2_rel": ((o - r).norm() / r.norm()).item()}
+        failed = not (worst < 2e-2)
     print(json.dumps(result))
+    if failed:
+        sys.stderr.write("bench.py: a layer of the GPU forward deviates from the CPU oracle by more than 2e-2\n")
+        raise SystemExit(1)
 
 
 if __name__ == "__main__":

@@ -80,8 +80,8 @@ int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int 
  * ------------------------------------------------------------------------------------------- */
 
 /* 1 if sequence length L is supported: a power of two in [128, 32768] (one LDS-resident transform per
- * row up to 1024, two half-length transforms per row for 2048 .. 16384, four LDS-resident
- * sub-transforms per row for 32768). */
+ * row up to 1024, two half-length transforms per row for 2048 .. 16384; at 32768 each of the two real signals
+ * of a row is convolved on its own in polyphase form, again as two LDS-resident half transforms). */
 int m2_fftconv_supported_seqlen(int L);
 
 /* Bytes of the opaque spectrum buffer for d channels and sequence length L (both filters): 16 d L, and 24 d L at
@@ -161,11 +161,16 @@ int m2_blockdiag_linear_layernorm_fwd(const void* x, const void* w, const float*
  * out = LayerNorm(e) in the same three forms as m2_layernorm_fwd (any may be NULL).
  * input_ids (B, L) int64; token_type_ids (B, L) int64 or NULL (all zero); pos_emb NULL when the model has no
  * position embeddings, else position_ids (B, L) int64 or NULL (positions 0 .. L-1 in every sequence).
- * Tables are fp32 row-major (rows, d); indices are not range-checked.  Needs d % 64 == 0, d <= 2048. */
+ * Tables are fp32 row-major: word_emb (vocab_size, d), type_emb (type_vocab_size, d), pos_emb (max_positions, d).
+ * An index outside its table (the reference's nn.Embedding raises there) never reads foreign memory: the kernel
+ * uses the nearest valid row instead and, when bad_index is not NULL, stores 1 to *bad_index (device memory, one
+ * int, which the caller zeroed before the call and reads after the stream has run).  Without position_ids the
+ * call fails with M2_ERR_ARG when L > max_positions.  Needs d % 64 == 0, d <= 2048. */
 int m2_embed_layernorm_fwd(const long long* input_ids, const long long* token_type_ids, const long long* position_ids,
-                           const float* word_emb, const float* type_emb, const float* pos_emb, const float* gamma,
-                           const float* beta, float eps, float* out_f32, void* out_bf16, float* out_channel_major,
-                           int B, int L, int d, void* stream);
+                           const float* word_emb, const float* type_emb, const float* pos_emb, int vocab_size,
+                           int type_vocab_size, int max_positions, const float* gamma, const float* beta, float eps,
+                           float* out_f32, void* out_bf16, float* out_channel_major, int* bad_index, int B, int L,
+                           int d, void* stream);
 
 #ifdef __cplusplus
 }

@@ -61,7 +61,8 @@ def _load() -> ctypes.CDLL:
     lib.m2_blockdiag_linear_layernorm_fwd.restype = c_int
     lib.m2_blockdiag_linear_layernorm_fwd.argtypes = [c_void_p] * 6 + [c_float] + [c_void_p] * 3 + [c_int] * 4 + [c_void_p]
     lib.m2_embed_layernorm_fwd.restype = c_int
-    lib.m2_embed_layernorm_fwd.argtypes = [c_void_p] * 8 + [c_float] + [c_void_p] * 3 + [c_int, c_int, c_int, c_void_p]
+    lib.m2_embed_layernorm_fwd.argtypes = ([c_void_p] * 6 + [c_int] * 3 + [c_void_p] * 2 + [c_float] + [c_void_p] * 4
+                                           + [c_int, c_int, c_int, c_void_p])
     return lib
 
 

@@ -464,6 +464,9 @@ struct LnShape {
 };
 // Where the rows come from when the kernel normalises embeddings instead of a matrix:
 // row m = word[ids[m]] + type[tt[m] or 0] (+ pos[pos_ids[m] or m % L]).
+// Every index is clamped into its table before it is used, so a bad id reads a valid row instead of
+// foreign memory; when that happens and `bad_index` is not null the kernel stores 1 there (plain vector
+// store; the caller cleared it before the launch and reads it afterwards to report the error).
 struct EmbedSource {
   const long long* ids;     // (M)
   const long long* tt;      // (M) or null: type 0
@@ -472,7 +475,16 @@ struct EmbedSource {
   const float* type;        // (type_vocab, d)
   const float* pos;         // (max_positions, d) or null: no position embeddings
   int L;
+  int vocab, type_vocab, max_positions;      // rows of the three tables
+  int* bad_index;           // or null
 };
+__device__ __forceinline__ long long clamp_index(long long i, int rows, bool& bad) {
+  if (i < 0 || i >= rows) {
+    bad = true;
+    return i < 0 ? 0 : rows - 1;
+  }
+  return i;
+}
 template <int PER, bool EMBED>
 __global__ __launch_bounds__(512) void layernorm_kernel(const float* __restrict__ x, EmbedSource src,
                                                         const float* __restrict__ gamma,
@@ -501,19 +513,22 @@ __global__ __launch_bounds__(512) void layernorm_kernel(const float* __restrict_
       const float* xr = x + (long)m * d;
       static_for<0, PER>([&](auto ii) { v[rr][decltype(ii)::value] = xr[lane + 64 * decltype(ii)::value]; });
     } else {
-      const float* wr = src.word + src.ids[m] * d;
-      const float* tr = src.type + (src.tt ? src.tt[m] : 0) * d;
+      bool bad = false;
+      const float* wr = src.word + clamp_index(src.ids[m], src.vocab, bad) * d;
+      const float* tr = src.type + (src.tt ? clamp_index(src.tt[m], src.type_vocab, bad) : 0) * d;
       static_for<0, PER>([&](auto ii) {
         constexpr int i = decltype(ii)::value;
         v[rr][i] = wr[lane + 64 * i] + tr[lane + 64 * i];
       });
       if (src.pos) {
-        const float* pr = src.pos + (src.pos_ids ? src.pos_ids[m] : (long long)(m % src.L)) * d;
+        const float* pr = src.pos + (src.pos_ids ? clamp_index(src.pos_ids[m], src.max_positions, bad)
+                                                 : (long long)(m % src.L)) * d;
         static_for<0, PER>([&](auto ii) {
           constexpr int i = decltype(ii)::value;
           v[rr][i] += pr[lane + 64 * i];
         });
       }
+      if (bad && src.bad_index && lane == 0) *src.bad_index = 1;
     }
   });
   static_for<0, RW>([&](auto rr_) {
@@ -975,15 +990,21 @@ extern "C" int m2_layernorm_fwd(const float* x, const float* gamma, const float*
 
 extern "C" int m2_embed_layernorm_fwd(const long long* input_ids, const long long* token_type_ids,
                                       const long long* position_ids, const float* word_emb, const float* type_emb,
-                                      const float* pos_emb, const float* gamma, const float* beta, float eps,
-                                      float* out_f32, void* out_bf16, float* out_channel_major, int B, int L, int d,
-                                      void* stream) {
+                                      const float* pos_emb, int vocab_size, int type_vocab_size, int max_positions,
+                                      const float* gamma, const float* beta, float eps, float* out_f32, void* out_bf16,
+                                      float* out_channel_major, int* bad_index, int B, int L, int d, void* stream) {
   if (!input_ids || !word_emb || !type_emb || !gamma || !beta)
     return set_error(M2_ERR_ARG, "m2_embed_layernorm_fwd: null pointer");
   if (B <= 0 || L <= 0 || d <= 0 || d % 64 != 0 || d > 2048)
     return set_error(M2_ERR_UNSUPPORTED, "m2_embed_layernorm_fwd: need B, L > 0 and d a multiple of 64 up to 2048 (B=%d L=%d d=%d)", B, L, d);
   if ((long)B * L > 0x7fffffffL) return set_error(M2_ERR_UNSUPPORTED, "m2_embed_layernorm_fwd: B * L = %ld does not fit an int", (long)B * L);
   if (position_ids && !pos_emb) return set_error(M2_ERR_ARG, "m2_embed_layernorm_fwd: position_ids without a position table");
-  const EmbedSource src{input_ids, token_type_ids, position_ids, word_emb, type_emb, pos_emb, L};
+  if (vocab_size <= 0 || type_vocab_size <= 0 || (pos_emb && max_positions <= 0))
+    return set_error(M2_ERR_ARG, "m2_embed_layernorm_fwd: table sizes must be positive (vocab=%d type_vocab=%d max_positions=%d)",
+                     vocab_size, type_vocab_size, max_positions);
+  if (pos_emb && !position_ids && L > max_positions)
+    return set_error(M2_ERR_ARG, "m2_embed_layernorm_fwd: sequence length %d exceeds the position table (%d rows)", L, max_positions);
+  const EmbedSource src{input_ids, token_type_ids, position_ids, word_emb, type_emb, pos_emb, L,
+                        vocab_size, type_vocab_size, max_positions, bad_index};
   return launch_layernorm<true>(nullptr, src, gamma, beta, eps, out_f32, out_bf16, out_channel_major, B * L, d, stream);
 }

@@ -45,6 +45,14 @@ class BertEmbeddings(nn.Module):
             self.register_buffer("position_ids", torch.arange(config.max_position_embeddings).expand((1, -1)))
         self.register_buffer("token_type_ids", torch.zeros(config.max_position_embeddings, dtype=torch.long),
                              persistent=False)
+        # set by the embedding kernel when an id lies outside its table (the kernel then reads the nearest valid
+        # row); `check_indices()` reads it.  Not part of the state dict.
+        self.register_buffer("_bad_index", torch.zeros(1, dtype=torch.int32), persistent=False)
+
+    def check_indices(self) -> None:
+        """Raises IndexError if a lookup since the last check used an id outside its table (nn.Embedding raises at
+        the lookup in the reference; here the kernel flags it and this call, which waits for the stream, reports)."""
+        ops.raise_on_bad_index(self._bad_index)
 
     def summed(self, input_ids=None, token_type_ids=None, position_ids=None, inputs_embeds=None,
                past_key_values_length: int = 0) -> torch.Tensor:
@@ -72,6 +80,8 @@ class BertEmbeddings(nn.Module):
             raise NotImplementedError("m2_amd is a forward/inference path: call .eval() first")
         o32, _, _ = self.forward_forms(input_ids, token_type_ids, position_ids, inputs_embeds, past_key_values_length,
                                        want_f32=True, want_bf16=False, want_channel_major=False)
+        if not torch.cuda.is_current_stream_capturing():
+            self.check_indices()
         return o32
 
     def forward_forms(self, input_ids=None, token_type_ids=None, position_ids=None, inputs_embeds=None,
@@ -94,7 +104,8 @@ class BertEmbeddings(nn.Module):
                 input_ids.contiguous(), None if token_type_ids is None else token_type_ids.expand(B, L).contiguous(), pos,
                 self.word_embeddings.weight.detach(), self.token_type_embeddings.weight.detach(),
                 self.position_embeddings.weight.detach() if self.use_positional_encodings else None, gamma, beta,
-                self.LayerNorm.eps, want_f32=want_f32, want_bf16=want_bf16, want_channel_major=want_channel_major)
+                self.LayerNorm.eps, want_f32=want_f32, want_bf16=want_bf16, want_channel_major=want_channel_major,
+                bad_index=self._bad_index)
         else:
             e = self.summed(input_ids, token_type_ids, position_ids, inputs_embeds, past_key_values_length).float()
             B, L, d = e.shape
@@ -204,8 +215,9 @@ class BertEncoder(nn.Module):
     """`use_hip_graph=True` captures the whole stack of layers into one HIP graph per input shape and replays
     it: at short sequence lengths the forward is launch-bound (about ten small kernels per layer) and the
     replay removes the per-launch host cost.  The graph holds device pointers of the weights (and of their
-    cached bf16 copies): it is dropped by `load_state_dict`, `.to()` / `.cuda()` and `reset_graphs()`; call
-    `reset_graphs()` after changing a parameter in place.  Nothing in the captured region uses a memset."""
+    cached bf16 copies): it is dropped by `load_state_dict` (of this module or of any module that contains
+    it), `.to()` / `.cuda()` and `reset_graphs()`; call `reset_graphs()` after changing a parameter in place.
+    Nothing in the captured region uses a memset."""
 
     OVERLAP_UPFRONT_MAX_L = 2048
 
@@ -227,6 +239,9 @@ class BertEncoder(nn.Module):
         #              blur per-kernel timings.
         self.overlap_filters = None
         self._filter_stream = None
+        # nn.Module.load_state_dict of a parent never calls a child's load_state_dict, but it does run the
+        # post hooks of every module it recursed into: new weights drop the captured graphs
+        self.register_load_state_dict_post_hook(BertEncoder._drop_graphs_after_load)
 
     # -- graph bookkeeping -------------------------------------------------------------------
     def reset_graphs(self) -> None:
@@ -236,9 +251,9 @@ class BertEncoder(nn.Module):
         self._graphs = {}
         return super()._apply(fn, *args, **kwargs)
 
-    def load_state_dict(self, *args, **kwargs):
-        self._graphs = {}
-        return super().load_state_dict(*args, **kwargs)
+    @staticmethod
+    def _drop_graphs_after_load(module, incompatible_keys) -> None:
+        module._graphs = {}
 
     # -- the fused schedule --------------------------------------------------------------------
     def _run_layers(self, h32: Optional[torch.Tensor], B: int, L: int, all_layers: bool,
@@ -391,6 +406,11 @@ class BertModel(nn.Module):
         self.embeddings = BertEmbeddings(config)
         self.encoder = BertEncoder(config, use_hip_graph=use_hip_graph)
         self.pooler = BertPooler(config) if add_pooling_layer else None
+        # True: every forward ends by reading the embedding kernel's out-of-range flag (one stream
+        # synchronisation) and raises IndexError like nn.Embedding would; False leaves the flag to
+        # `embeddings.check_indices()`.  The embedding tables are part of the captured graph too:
+        self.validate_ids = True
+        self.register_load_state_dict_post_hook(lambda module, keys: module.encoder.reset_graphs())
 
     def get_input_embeddings(self):
         return self.embeddings.word_embeddings
@@ -439,6 +459,8 @@ class BertModel(nn.Module):
                     dst.copy_(src)
             graph.replay()
             outs = [o.clone() for o in static_out]
+        if self.validate_ids and not torch.cuda.is_current_stream_capturing():
+            self.embeddings.check_indices()
         enc = [o.view(B, L, -1) for o in outs]
         pooled = None
         if self.pooler is not None:

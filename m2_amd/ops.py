@@ -199,9 +199,13 @@ def layernorm(x: Tensor, gamma: Tensor, beta: Tensor, eps: float, want_f32: bool
 
 def embed_layernorm(input_ids: Tensor, token_type_ids: Optional[Tensor], position_ids: Optional[Tensor], word_emb: Tensor,
                     type_emb: Tensor, pos_emb: Optional[Tensor], gamma: Tensor, beta: Tensor, eps: float,
-                    want_f32: bool = True, want_bf16: bool = False, want_channel_major: bool = False):
+                    want_f32: bool = True, want_bf16: bool = False, want_channel_major: bool = False,
+                    bad_index: Optional[Tensor] = None):
     """LayerNorm(word_emb[ids] + type_emb[token_type_ids or 0] (+ pos_emb[position_ids or 0..L-1])) for ids (B, L)
-    -> (f32 (B*L, d) | None, bf16 (B*L, d) | None, f32 (d, B*L) | None)."""
+    -> (f32 (B*L, d) | None, bf16 (B*L, d) | None, f32 (d, B*L) | None).
+
+    An index outside its table never reads out of bounds (the kernel takes the nearest valid row); `bad_index`,
+    a zeroed int32 GPU tensor of one element, receives 1 when that happened: see `raise_on_bad_index`."""
     B, L = input_ids.shape
     d = word_emb.shape[1]
     _require(input_ids, "input_ids", torch.int64)
@@ -219,15 +223,27 @@ def embed_layernorm(input_ids: Tensor, token_type_ids: Optional[Tensor], positio
         if pos_emb is None:
             raise ValueError("position_ids given but the model has no position embeddings")
         _require(position_ids, "position_ids", torch.int64, (B, L))
+    if bad_index is not None:
+        _require(bad_index, "bad_index", torch.int32, (1,))
     M = B * L
     dev = input_ids.device
     o32 = torch.empty(M, d, dtype=torch.float32, device=dev) if want_f32 else None
     o16 = torch.empty(M, d, dtype=torch.bfloat16, device=dev) if want_bf16 else None
     ot = torch.empty(d, M, dtype=torch.float32, device=dev) if want_channel_major else None
     check(lib.m2_embed_layernorm_fwd(_ptr(input_ids), _ptr(token_type_ids), _ptr(position_ids), _ptr(word_emb),
-                                     _ptr(type_emb), _ptr(pos_emb), _ptr(gamma), _ptr(beta), float(eps), _ptr(o32),
-                                     _ptr(o16), _ptr(ot), B, L, d, _stream()))
+                                     _ptr(type_emb), _ptr(pos_emb), word_emb.shape[0], type_emb.shape[0],
+                                     0 if pos_emb is None else pos_emb.shape[0], _ptr(gamma), _ptr(beta), float(eps),
+                                     _ptr(o32), _ptr(o16), _ptr(ot), _ptr(bad_index), B, L, d, _stream()))
     return o32, o16, ot
+
+
+def raise_on_bad_index(bad_index: Tensor) -> None:
+    """Reads the flag `embed_layernorm` sets (this waits for the stream) and raises IndexError, as nn.Embedding
+    does in the reference, when a token, token-type or position id lay outside its table."""
+    if int(bad_index.item()) != 0:
+        bad_index.zero_()
+        raise IndexError("index out of range in the embedding lookup: a token id, token-type id or position id "
+                         "lies outside its table (the output of this forward used the nearest valid rows)")
 
 
 def blockdiag_linear_layernorm_supported(in_features: int, out_features: int, nblocks: int) -> bool:

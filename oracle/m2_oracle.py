@@ -8,7 +8,11 @@ as the checker; nothing in the shipped `m2_amd` package imports, calls or falls 
 Every function takes plain tensors or a flat ``{name: tensor}`` state dict whose keys are the
 reference's own parameter / buffer names, so that the same weights can be loaded into the HIP
 modules with ``load_state_dict`` and handed to this file unchanged.  All arithmetic runs in the
-dtype of the tensors handed in (fp32 for parity runs, fp64 when a test wants a tighter pin).
+dtype of the tensors handed in (fp32 for parity runs, fp64 when a test wants a tighter pin).  The functions
+are plain torch ops with the reference's own expressions and dtype flow (`.to(k.dtype)` before the FFT,
+`bias.to(out.dtype)` in the structured linear), so a test may also run them on GPU tensors under
+`torch.autocast("cuda", dtype=torch.bfloat16)` to obtain the reference's mixed-precision numerics as PyTorch
+itself defines them.
 
 What pins each function (tests/test_oracle_*.py; no reference code is imported or run):
 
@@ -44,23 +48,6 @@ Tensor = torch.Tensor
 StateDict = Dict[str, Tensor]
 
 
-def bf16_round(x: Tensor) -> Tensor:
-    """Round to bfloat16 and back: one autocast rounding point."""
-    return x.to(torch.bfloat16).to(x.dtype)
-
-
-def _ident(x: Tensor) -> Tensor:
-    return x
-
-
-def _rd(emulate_autocast: bool):
-    """`emulate_autocast=True` restates the reference's *CUDA autocast(bf16)* numerics on the CPU: every
-    tensor the reference would hold in bf16 is rounded to bf16 (matmuls still accumulate in fp32, as
-    the GPU does).  It is a yardstick for how far bf16 execution itself moves the result away from
-    the fp32 path; parity is always judged against the fp32 oracle (emulate_autocast=False)."""
-    return bf16_round if emulate_autocast else _ident
-
-
 # --------------------------------------------------------------------------------------
 # HyenaFilter pieces
 # --------------------------------------------------------------------------------------
@@ -93,7 +80,7 @@ def modulation_deltas(d_model: int, fast_decay_pct: float = 0.3, slow_decay_pct:
 
 
 def hyena_filter_taps(sd: StateDict, prefix: str, L: int, rev: bool = False,
-                      w_mod: float = 1.0, shift: float = 0.0, emulate_autocast: bool = False) -> Tensor:
+                      w_mod: float = 1.0, shift: float = 0.0) -> Tensor:
     """Implicit filter h (1, L, d): sin-MLP over the positional embedding, then decay.
 
     bert/src/mm/hyena_utils.py:201-217 (`filter` / `filter_rev`), :50-63 (`Sin`),
@@ -104,13 +91,12 @@ def hyena_filter_taps(sd: StateDict, prefix: str, L: int, rev: bool = False,
     z = sd[prefix + "pos_emb.z"][:, :L]
     t = sd[prefix + "pos_emb.t"][:, :L]
     freq = sd[prefix + "implicit_filter.1.freq"]
-    rd = _rd(emulate_autocast)
     h = z
     idx = 0
     while (mlp + f"{idx}.weight") in sd:
         w = sd[mlp + f"{idx}.weight"]
         b = sd.get(mlp + f"{idx}.bias")
-        h = rd(F.linear(rd(h), rd(w), None if b is None else rd(b)))
+        h = F.linear(h, w, None if b is None else b)
         if (mlp + f"{idx + 2}.weight") in sd:      # every Linear but the last is followed by Sin
             h = torch.sin(w_mod * freq * h)
         idx += 2
@@ -163,20 +149,18 @@ def short_conv(u: Tensor, weight: Tensor, bias: Tensor) -> Tensor:
 
 
 def mixer_filters(sd: StateDict, prefix: str, L: int, bidirectional: bool = True,
-                  residual_long_conv: bool = True, w_mod: float = 1.0, emulate_autocast: bool = False):
+                  residual_long_conv: bool = True, w_mod: float = 1.0):
     """The (up to) four tap sets of one mixer, each (d, L): k, k_rev, k2, k2_rev."""
     out = []
     for fn in (["filter_fn."] + (["filter_fn2."] if residual_long_conv else [])):
-        k = hyena_filter_taps(sd, prefix + fn, L, rev=False, w_mod=w_mod,
-                              emulate_autocast=emulate_autocast)[0].transpose(0, 1)
-        kr = hyena_filter_taps(sd, prefix + fn, L, rev=True, w_mod=w_mod,
-                               emulate_autocast=emulate_autocast)[0].transpose(0, 1) if bidirectional else None
+        k = hyena_filter_taps(sd, prefix + fn, L, rev=False, w_mod=w_mod)[0].transpose(0, 1)
+        kr = hyena_filter_taps(sd, prefix + fn, L, rev=True, w_mod=w_mod)[0].transpose(0, 1) if bidirectional else None
         out += [k, kr]
     return out
 
 
 def mixer_forward(sd: StateDict, prefix: str, u: Tensor, bidirectional: bool = True,
-                  residual_long_conv: bool = True, w_mod: float = 1.0, emulate_autocast: bool = False,
+                  residual_long_conv: bool = True, w_mod: float = 1.0,
                   training_additions: bool = False) -> Tensor:
     """MonarchMixerSequenceMixing.forward in eval mode, u (B, L, d) -> (B, L, d).
 
@@ -186,24 +170,23 @@ def mixer_forward(sd: StateDict, prefix: str, u: Tensor, bidirectional: bool = T
     :150-151) do nothing in eval mode.
     """
     B, L, d = u.shape
-    rd = _rd(emulate_autocast)
     if training_additions:
         u = F.layer_norm(u, (d,), sd[prefix + "layernorm.weight"], sd[prefix + "layernorm.bias"], 1e-5)
     u_orig = u
-    x = rd(F.linear(rd(u), rd(sd[prefix + "in_linear.weight"]), rd(sd[prefix + "in_linear.bias"])))
+    x = F.linear(u, sd[prefix + "in_linear.weight"], sd[prefix + "in_linear.bias"])
     x = x.transpose(1, 2)                                             # (B, 3d, L)
-    uc = rd(short_conv(x, rd(sd[prefix + "short_filter.weight"]), rd(sd[prefix + "short_filter.bias"])))
+    uc = short_conv(x, sd[prefix + "short_filter.weight"], sd[prefix + "short_filter.bias"])
     x1, x2, v = uc.split(d, dim=1)
-    v = rd(v * x1)
-    filt = mixer_filters(sd, prefix, L, bidirectional, residual_long_conv, w_mod, emulate_autocast)
-    y = rd(hyena_filter_forward(v, L, filt[0], filt[1], sd[prefix + "filter_fn.bias"][None, :, None]))
-    y = rd(y * x2)
+    v = v * x1
+    filt = mixer_filters(sd, prefix, L, bidirectional, residual_long_conv, w_mod)
+    y = hyena_filter_forward(v, L, filt[0], filt[1], sd[prefix + "filter_fn.bias"][None, :, None])
+    y = y * x2
     if residual_long_conv:
         yu = hyena_filter_forward(u_orig.transpose(1, 2), L, filt[2], filt[3],
                                   sd[prefix + "filter_fn2.bias"][None, :, None])
         y = y + yu
     y = y.transpose(1, 2)
-    return rd(F.linear(rd(y), rd(sd[prefix + "out_linear.weight"]), rd(sd[prefix + "out_linear.bias"])))
+    return F.linear(y, sd[prefix + "out_linear.weight"], sd[prefix + "out_linear.bias"])
 
 
 # --------------------------------------------------------------------------------------
@@ -234,7 +217,7 @@ def blockdiag_linear(x: Tensor, weight: Tensor, bias: Optional[Tensor], in_featu
 
 
 def glu_mlp_forward(sd: StateDict, prefix: str, x: Tensor, intermediate_size: int,
-                    layer_norm_eps: float = 1e-12, emulate_autocast: bool = False) -> Tensor:
+                    layer_norm_eps: float = 1e-12) -> Tensor:
     """BertGatedLinearUnitMLP.forward with BlockdiagLinear layers, x (B, L, d).
 
     bert/src/bert_layers.py:482-508: h = gated_layers(x); gelu_erf(h[..., :I]) * h[..., I:];
@@ -242,29 +225,28 @@ def glu_mlp_forward(sd: StateDict, prefix: str, x: Tensor, intermediate_size: in
     """
     d = x.shape[-1]
     I = intermediate_size
-    rd = _rd(emulate_autocast)
-    h = rd(blockdiag_linear(rd(x), rd(sd[prefix + "gated_layers.weight"]), None, d, 2 * I))
-    a = rd(rd(F.gelu(h[..., :I])) * h[..., I:])
-    o = rd(rd(blockdiag_linear(a, rd(sd[prefix + "wo.weight"]), None, I, d)) + rd(sd[prefix + "wo.bias"]))
-    return F.layer_norm(rd(o + x), (d,), sd[prefix + "layernorm.weight"], sd[prefix + "layernorm.bias"],
+    h = blockdiag_linear(x, sd[prefix + "gated_layers.weight"], None, d, 2 * I)
+    a = F.gelu(h[..., :I]) * h[..., I:]
+    o = blockdiag_linear(a, sd[prefix + "wo.weight"], sd[prefix + "wo.bias"], I, d)
+    return F.layer_norm(o + x, (d,), sd[prefix + "layernorm.weight"], sd[prefix + "layernorm.bias"],
                         layer_norm_eps)
 
 
 # --------------------------------------------------------------------------------------
 # Layer / encoder / embeddings
 # --------------------------------------------------------------------------------------
-def layer_forward(sd: StateDict, prefix: str, x: Tensor, cfg, emulate_autocast: bool = False) -> Tensor:
+def layer_forward(sd: StateDict, prefix: str, x: Tensor, cfg) -> Tensor:
     """BertLayer.forward, M2 branch: mlp(attention(x)); no norm/residual around the mixer.
 
     bert/src/bert_layers.py:575-599.
     """
     a = mixer_forward(sd, prefix + "attention.", x, cfg.bidirectional, cfg.residual_long_conv,
-                      cfg.hyena_w_mod, emulate_autocast, getattr(cfg, "hyena_training_additions", False))
-    return glu_mlp_forward(sd, prefix + "mlp.", a, cfg.intermediate_size, cfg.layer_norm_eps, emulate_autocast)
+                      cfg.hyena_w_mod, getattr(cfg, "hyena_training_additions", False))
+    return glu_mlp_forward(sd, prefix + "mlp.", a, cfg.intermediate_size, cfg.layer_norm_eps)
 
 
 def encoder_forward(sd: StateDict, prefix: str, x: Tensor, attention_mask: Optional[Tensor], cfg,
-                    output_all_encoded_layers: bool = False, emulate_autocast: bool = False) -> List[Tensor]:
+                    output_all_encoded_layers: bool = False) -> List[Tensor]:
     """BertEncoder.forward, M2 branch (bert/src/bert_layers.py:691-813).
 
     The attention mask never reaches an M2 layer (:577, :721-726): pad positions are
@@ -272,7 +254,7 @@ def encoder_forward(sd: StateDict, prefix: str, x: Tensor, attention_mask: Optio
     """
     outs = []
     for i in range(cfg.num_hidden_layers):
-        x = layer_forward(sd, f"{prefix}layer.{i}.", x, cfg, emulate_autocast)
+        x = layer_forward(sd, f"{prefix}layer.{i}.", x, cfg)
         if output_all_encoded_layers:
             outs.append(x)
     if not output_all_encoded_layers:
@@ -306,15 +288,14 @@ def pooler_forward(sd: StateDict, prefix: str, hidden: Tensor, mask: Optional[Te
 
 
 def model_forward(sd: StateDict, input_ids: Tensor, attention_mask: Optional[Tensor], cfg,
-                  prefix: str = "", emulate_autocast: bool = False, pooled: bool = False):
+                  prefix: str = "", pooled: bool = False):
     """BertModel.forward: embeddings -> encoder, last hidden state (B, L, d); with pooled=True also the
     pooler's output, as a pair.
 
     bert/src/bert_layers.py:948-1010.
     """
     x = embeddings_forward(sd, prefix + "embeddings.", input_ids, cfg)
-    seq = encoder_forward(sd, prefix + "encoder.", x, attention_mask, cfg,
-                          emulate_autocast=emulate_autocast)[-1]
+    seq = encoder_forward(sd, prefix + "encoder.", x, attention_mask, cfg)[-1]
     if not pooled:
         return seq
     if attention_mask is None:

@@ -340,18 +340,6 @@ def test_embeddings_gather_and_layernorm():
     assert not torch.allclose(O.embeddings_forward(sd, "embeddings.", ids, cfg, tt), got)
 
 
-def test_autocast_emulation_is_a_small_perturbation_of_fp32():
-    """The bf16-emulating mode is only a yardstick; it must stay close to the fp32 path on one layer."""
-    import m2_amd
-    cfg = m2_amd.M2BertConfig(hidden_size=64, intermediate_size=128, num_hidden_layers=1, vocab_size=64).with_seq_len(64)
-    sd = m2_amd.seeded_state_dict(cfg, 8)
-    ids = torch.randint(0, 64, (2, 64), generator=torch.Generator().manual_seed(3))
-    a = O.model_forward(sd, ids, None, cfg)
-    b = O.model_forward(sd, ids, None, cfg, emulate_autocast=True)
-    rel = ((a - b).norm() / a.norm()).item()
-    assert 1e-4 < rel < 2e-2
-
-
 def test_mixer_training_additions_is_a_pre_layernorm_seen_by_both_convolutions():
     """hyena_training_additions in eval mode: the input LayerNorm (eps 1e-5) feeds the projections AND the
     residual long convolution (monarch_mixer_sequence_mixer.py:102-107); everything else is unchanged.  Checked
@@ -363,14 +351,14 @@ def test_mixer_training_additions_is_a_pre_layernorm_seen_by_both_convolutions()
     cfg.hyena_training_additions = True
     sd = {k: v.double() for k, v in m2_amd.seeded_state_dict(cfg, 5, std=0.3, what="mixer").items()}
     u = torch.randn(2, 64, 64, dtype=torch.float64, generator=torch.Generator().manual_seed(2)) * 3 + 1.5
-    got = O.mixer_forward(sd, "", u, True, True, 1.0, False, True)
+    got = O.mixer_forward(sd, "", u, True, True, 1.0, True)
     mu = u.mean(-1, keepdim=True)
     var = ((u - mu) ** 2).mean(-1, keepdim=True)
     un = (u - mu) / torch.sqrt(var + 1e-5) * sd["layernorm.weight"] + sd["layernorm.bias"]
-    want = O.mixer_forward(sd, "", un, True, True, 1.0, False, False)
+    want = O.mixer_forward(sd, "", un, True, True, 1.0, False)
     assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
     # the residual convolution must see the normalised input: feeding it the raw input changes the result
-    plain = O.mixer_forward(sd, "", u, True, True, 1.0, False, False)
+    plain = O.mixer_forward(sd, "", u, True, True, 1.0, False)
     assert (got - plain).abs().max() > 1e-3
 
 
