@@ -72,6 +72,20 @@ size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int order);
 int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order, int emb_dim,
                         float w_mod, float shift, float* workspace, float* taps, void* stream);
 
+/* The same computation as m2_hyena_filter_fwd without the workspace argument.  This entry point has no
+ * counterpart in the reference: it exists for callers that cannot allocate device memory around the call (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The intermediate activations
+ * go through a device array of M2_HYENA_FILTER_STATIC_SCRATCH_BYTES that is part of the library itself (every GPU
+ * the library runs on holds one copy until the process ends); the call allocates and frees nothing.  Limit:
+ * m2_hyena_filter_workspace_bytes(nfilters, L, order) must not exceed that size, i.e. nfilters * L <= 16384 (both
+ * filters of a mixer up to L = 8192); beyond it the call fails with M2_ERR_UNSUPPORTED.  All calls on one GPU share
+ * the array: two such calls whose kernels may overlap on the same GPU (different streams, or different host threads
+ * on different streams) race; calls on one stream are ordered and safe.  The first call on a device looks up the
+ * array's device address (hipGetSymbolAddress): make that call outside a stream capture. */
+#define M2_HYENA_FILTER_STATIC_SCRATCH_BYTES (16u << 20)
+int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order,
+                               int emb_dim, float w_mod, float shift, float* taps, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Long convolution: filter spectra and the fused mixer core.
  * Stand in for: bert/src/mm/hyena_utils.py:16-42 (fftconv_ref), :219-248 (HyenaFilter.forward) and

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libm2_amd.so")
 
 M2_DTYPE_F32 = 0
 M2_DTYPE_BF16 = 1
+M2_HYENA_FILTER_STATIC_SCRATCH_BYTES = 16 << 20
 
 
 class HyenaFilterParams(ctypes.Structure):
@@ -37,6 +38,9 @@ def _load() -> ctypes.CDLL:
     lib.m2_hyena_filter_fwd.restype = c_int
     lib.m2_hyena_filter_fwd.argtypes = [POINTER(HyenaFilterParams), c_int, c_int, c_int, c_int, c_int, c_float,
                                         c_float, c_void_p, c_void_p, c_void_p]
+    lib.m2_hyena_filter_fwd_static.restype = c_int
+    lib.m2_hyena_filter_fwd_static.argtypes = [POINTER(HyenaFilterParams), c_int, c_int, c_int, c_int, c_int, c_float,
+                                               c_float, c_void_p, c_void_p]
     lib.m2_fftconv_supported_seqlen.restype = c_int
     lib.m2_fftconv_supported_seqlen.argtypes = [c_int]
     lib.m2_filter_spectrum_bytes.restype = c_size_t
@@ -68,7 +72,7 @@ def _load() -> ctypes.CDLL:
 
 lib = _load()
 
-EXPORTS = ["m2_version", "m2_last_error", "m2_hyena_filter_workspace_bytes", "m2_hyena_filter_fwd",
+EXPORTS = ["m2_version", "m2_last_error", "m2_hyena_filter_workspace_bytes", "m2_hyena_filter_fwd", "m2_hyena_filter_fwd_static",
            "m2_fftconv_supported_seqlen", "m2_filter_spectrum_bytes", "m2_filter_spectrum_fwd", "m2_mixer_core_fwd",
            "m2_fftconv_fwd", "m2_blockdiag_glu_fwd", "m2_blockdiag_linear_fwd", "m2_layernorm_fwd",
            "m2_embed_layernorm_fwd", "m2_blockdiag_linear_layernorm_supported", "m2_blockdiag_linear_layernorm_fwd"]

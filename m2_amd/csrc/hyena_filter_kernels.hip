@@ -16,6 +16,8 @@
 // stores the taps channel-major, forward taps at [0, L) and reverse taps mirrored into [L, 2L).
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "m2_internal.h"
 
 namespace m2 {
@@ -265,26 +267,26 @@ extern "C" size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int order
   return (size_t)2 * nfilters * L * order * sizeof(float);
 }
 
-extern "C" int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order,
-                                   int emb_dim, float w_mod, float shift, float* workspace, float* taps,
-                                   void* stream) {
-  if (!params || !workspace || !taps) return set_error(M2_ERR_ARG, "m2_hyena_filter_fwd: null pointer");
+// Shared by the two entry points: validation and the two launches, `workspace` holding the h3 hi / lo parts.
+static int hyena_filter_launch(const char* who, const m2_hyena_filter_params* params, int nfilters, int L, int d,
+                               int order, int emb_dim, float w_mod, float shift, void* workspace, float* taps,
+                               void* stream) {
   if (nfilters < 1 || nfilters > kMaxFilters)
-    return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: nfilters=%d not in [1, %d]", nfilters, kMaxFilters);
-  if (order != kOrder) return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: order=%d, only 128 is built", order);
+    return set_error(M2_ERR_UNSUPPORTED, "%s: nfilters=%d not in [1, %d]", who, nfilters, kMaxFilters);
+  if (order != kOrder) return set_error(M2_ERR_UNSUPPORTED, "%s: order=%d, only 128 is built", who, order);
   if (emb_dim < 3 || emb_dim > kMaxEmb)
-    return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: emb_dim=%d not in [3, %d]", emb_dim, kMaxEmb);
+    return set_error(M2_ERR_UNSUPPORTED, "%s: emb_dim=%d not in [3, %d]", who, emb_dim, kMaxEmb);
   if (L <= 0 || L % kPosTile != 0)
-    return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: L=%d must be a positive multiple of %d", L, kPosTile);
-  if (d <= 0 || d % 64 != 0) return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd: d=%d must be a positive multiple of 64", d);
+    return set_error(M2_ERR_UNSUPPORTED, "%s: L=%d must be a positive multiple of %d", who, L, kPosTile);
+  if (d <= 0 || d % 64 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: d=%d must be a positive multiple of 64", who, d);
   FilterBatch fb;
   for (int f = 0; f < kMaxFilters; ++f) {
     const m2_hyena_filter_params& p = params[f < nfilters ? f : 0];
     if (!p.z || !p.t || !p.freq || !p.deltas || !p.w0 || !p.b0 || !p.w1 || !p.b1 || !p.w2 || !p.b2 || !p.w3)
-      return set_error(M2_ERR_ARG, "m2_hyena_filter_fwd: filter %d has a null forward-MLP pointer", f);
+      return set_error(M2_ERR_ARG, "%s: filter %d has a null forward-MLP pointer", who, f);
     const bool rev = p.rw0 != nullptr;
     if (rev && (!p.rb0 || !p.rw1 || !p.rb1 || !p.rw2 || !p.rb2 || !p.rw3))
-      return set_error(M2_ERR_ARG, "m2_hyena_filter_fwd: filter %d has a partly null reverse MLP", f);
+      return set_error(M2_ERR_ARG, "%s: filter %d has a partly null reverse MLP", who, f);
     fb.f[f].z = p.z; fb.f[f].t = p.t; fb.f[f].freq = p.freq; fb.f[f].deltas = p.deltas;
     fb.f[f].mlp[0] = MlpPtrs{p.w0, p.b0, p.w1, p.b1, p.w2, p.b2, p.w3};
     fb.f[f].mlp[1] = rev ? MlpPtrs{p.rw0, p.rb0, p.rw1, p.rb1, p.rw2, p.rb2, p.rw3}
@@ -299,4 +301,68 @@ extern "C" int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfi
   hipLaunchKernelGGL(project_kernel, dim3((L + kPosPerWg - 1) / kPosPerWg, (d + 127) / 128, 2 * nfilters), dim3(256), 0, s, fb, L, d, shift,
                      h_hi, h_lo, taps);
   return check_launch("hyena project_kernel");
+}
+
+extern "C" int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order,
+                                   int emb_dim, float w_mod, float shift, float* workspace, float* taps,
+                                   void* stream) {
+  if (!params || !workspace || !taps) return set_error(M2_ERR_ARG, "m2_hyena_filter_fwd: null pointer");
+  return hyena_filter_launch("m2_hyena_filter_fwd", params, nfilters, L, d, order, emb_dim, w_mod, shift, workspace,
+                             taps, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same computation for callers that cannot allocate a workspace: the h3 hi / lo parts go through a
+// device array that is part of the library's code object.  Every GPU the library runs on holds its own copy
+// of the array at its own address until the process ends; in host code the array's NAME is only a stand-in
+// for the symbol, so its device address is looked up once per device (hipGetSymbolAddress) and only that
+// address is ever handed to a kernel.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[M2_HYENA_FILTER_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};      // device address of `scratch` on device i, once looked up
+
+// Device address of the static scratch array on the current device (looked up on the first call per device).
+int static_scratch_for_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "m2_hyena_filter_fwd_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return set_error(M2_ERR_UNSUPPORTED, "m2_hyena_filter_fwd_static: device index %d beyond %d", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return set_error(M2_ERR_LAUNCH, "m2_hyena_filter_fwd_static: hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                       hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return M2_OK;
+}
+}  // namespace
+
+extern "C" int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order,
+                                          int emb_dim, float w_mod, float shift, float* taps, void* stream) {
+  if (!params || !taps) return set_error(M2_ERR_ARG, "m2_hyena_filter_fwd_static: null pointer");
+  if (nfilters < 1 || L <= 0 || order <= 0)
+    return set_error(M2_ERR_ARG, "m2_hyena_filter_fwd_static: sizes must be positive (nfilters=%d L=%d order=%d)", nfilters, L, order);
+  const size_t need = m2_hyena_filter_workspace_bytes(nfilters, L, order);
+  if (need > (size_t)M2_HYENA_FILTER_STATIC_SCRATCH_BYTES)
+    return set_error(M2_ERR_UNSUPPORTED,
+                     "m2_hyena_filter_fwd_static: nfilters=%d, L=%d needs %zu bytes of scratch, the static array holds %zu "
+                     "(nfilters * L <= %zu); use m2_hyena_filter_fwd with a caller workspace",
+                     nfilters, L, need, (size_t)M2_HYENA_FILTER_STATIC_SCRATCH_BYTES,
+                     (size_t)M2_HYENA_FILTER_STATIC_SCRATCH_BYTES / (2 * kOrder * sizeof(float)));
+  void* ptr = nullptr;
+  int rc = static_scratch_for_current_device(&ptr);
+  if (rc) return rc;
+  // hidden_kernel writes every h3 element project_kernel reads in the same call, so nothing left by an earlier
+  // (possibly longer) call is ever read and nothing needs clearing
+  return hyena_filter_launch("m2_hyena_filter_fwd_static", params, nfilters, L, d, order, emb_dim, w_mod, shift, ptr,
+                             taps, stream);
 }

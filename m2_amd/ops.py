@@ -53,11 +53,13 @@ def fftconv_supported(L: int) -> bool:
 
 # ------------------------------------------------------------------------------------------------
 def hyena_filter_taps(filters: Sequence[dict], L: int, d: int, order: int, emb_dim: int, w_mod: float = 1.0,
-                      shift: float = 0.0) -> Tensor:
+                      shift: float = 0.0, static_scratch: bool = False, out: Optional[Tensor] = None) -> Tensor:
     """Bidirectional taps (nfilters, d, 2L) fp32 of `filters`.
 
     Each entry is a dict with fp32 GPU tensors: z (>=L, emb), t (>=L), freq (order), deltas (d),
     `fwd` = [w0, b0, w1, b1, w2, b2, w3] and optionally `rev` = the same seven of the reverse MLP.
+    `static_scratch=True` takes the library's allocation-free entry point (m2_hyena_filter_fwd_static: no
+    workspace tensor, nfilters * L <= 16384); with `out` given as well nothing is allocated at all.
     """
     nf = len(filters)
     arr = (HyenaFilterParams * nf)()
@@ -87,9 +89,17 @@ def hyena_filter_taps(filters: Sequence[dict], L: int, d: int, order: int, emb_d
                 keep.append(w)
                 setattr(arr[i], n, w.data_ptr())
     dev = keep[0].device
+    if out is None:
+        taps = torch.empty(nf, d, 2 * L, dtype=torch.float32, device=dev)
+    else:
+        _require(out, "out", torch.float32, (nf, d, 2 * L))
+        taps = out
+    if static_scratch:
+        check(lib.m2_hyena_filter_fwd_static(arr, nf, L, d, order, emb_dim, float(w_mod), float(shift), _ptr(taps),
+                                             _stream()))
+        return taps
     ws_bytes = lib.m2_hyena_filter_workspace_bytes(nf, L, order)
     workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
-    taps = torch.empty(nf, d, 2 * L, dtype=torch.float32, device=dev)
     check(lib.m2_hyena_filter_fwd(arr, nf, L, d, order, emb_dim, float(w_mod), float(shift), _ptr(workspace),
                                   _ptr(taps), _stream()))
     return taps
