@@ -151,6 +151,19 @@ int m2_blockdiag_glu_fwd(const void* x, const void* w, void* out, int M, int in_
 int m2_blockdiag_linear_fwd(const void* x, const void* w, const float* bias, const void* residual, void* out, int M,
                             int in_features, int out_features, int nblocks, int out_dtype, void* stream);
 
+/* The whole GLU MLP up to the LayerNorm input in one kernel, the (M, 2I) and (M, I) intermediates never leaving the
+ * chip:  out = blockdiag_multiply(gelu_erf(h[:, :I]) * h[:, I:], w_out) (+ bias) (+ residual),
+ * h = blockdiag_multiply(x, w_gated)  (bert/src/bert_layers.py:482-506: gated_layers, act, wo, residual).  Same
+ * arithmetic as m2_blockdiag_glu_fwd followed by m2_blockdiag_linear_fwd (bf16 operands, fp32 accumulation, the
+ * gated values rounded to bf16 between the two products).  x (M, in_features) bf16; w_gated (nblocks, 2I/nblocks,
+ * in/nblocks) bf16; w_out (nblocks, in/nblocks, I/nblocks) bf16; bias (in_features) fp32 or NULL; residual
+ * (M, in_features) bf16 or NULL; out (M, in_features) of out_dtype.  m2_mlp_fused_supported returns 1 for the shapes
+ * the kernel is built for (nblocks == 4, in_features == 768, intermediate % 128 == 0); for others the entry point
+ * returns M2_ERR_UNSUPPORTED and the caller uses the two separate entry points. */
+int m2_mlp_fused_supported(int in_features, int intermediate, int nblocks);
+int m2_mlp_fused_fwd(const void* x, const void* w_gated, const void* w_out, const float* bias, const void* residual,
+                     void* out, int M, int in_features, int intermediate, int nblocks, int out_dtype, void* stream);
+
 /* LayerNorm over the last dimension of x (M, d) fp32 (torch.nn.LayerNorm semantics, biased variance,
  * eps inside the root; bert/src/bert_layers.py:478-479,506 and :185-186,247).  Any of the three
  * outputs may be NULL: out_f32 (M, d) fp32, out_bf16 (M, d) bf16, out_channel_major (d, M) fp32 (the

@@ -138,7 +138,8 @@ class MonarchMixerSequenceMixing(nn.Module):
                 u2, u16, u_cm = self.pre_norm(u2.float().contiguous(), want_f32=not low, want_bf16=low)
                 if low:
                     u2 = u16
-            xproj = torch.mm(w_in, u2.to(act).t())                                      # (3d, B*L), bias added in the core
+            xproj = torch.empty(3 * d, B * L, dtype=act, device=u.device)               # (3d, B*L), bias added in the core
+            torch.mm(u2.to(act), w_in.t(), out=xproj.t())
             if u_cm is None and self.residual_long_conv:
                 u_cm = u2.float().t().contiguous()                                       # (d, B*L)
             if not self.residual_long_conv:

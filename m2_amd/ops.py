@@ -192,6 +192,35 @@ def blockdiag_linear(x: Tensor, w: Tensor, bias: Optional[Tensor] = None, residu
     return out
 
 
+def mlp_fused_supported(in_features: int, intermediate: int, nblocks: int) -> bool:
+    return bool(lib.m2_mlp_fused_supported(int(in_features), int(intermediate), int(nblocks)))
+
+
+def mlp_fused(x: Tensor, w_gated: Tensor, w_out: Tensor, bias: Optional[Tensor] = None, residual: Optional[Tensor] = None,
+              out_dtype=torch.float32, out: Optional[Tensor] = None) -> Tensor:
+    """blockdiag(gelu_erf(h[:, :I]) * h[:, I:], w_out) (+ bias) (+ residual) with h = blockdiag(x, w_gated), one kernel.
+    x (M, d) bf16, w_gated (nb, 2I/nb, d/nb) bf16, w_out (nb, d/nb, I/nb) bf16."""
+    M, d = x.shape
+    nb, q, p = w_gated.shape
+    _require(x, "x", torch.bfloat16)
+    _require(w_gated, "w_gated", torch.bfloat16)
+    I = nb * q // 2
+    _require(w_out, "w_out", torch.bfloat16, (nb, d // nb, I // nb))
+    if nb * p != d:
+        raise ValueError(f"x has {d} features, w_gated expects {nb}*{p}")
+    if bias is not None:
+        _require(bias, "bias", torch.float32, (d,))
+    if residual is not None:
+        _require(residual, "residual", torch.bfloat16, (M, d))
+    if out is None:
+        out = torch.empty(M, d, dtype=out_dtype, device=x.device)
+    else:
+        _require(out, "out", out_dtype, (M, d))
+    check(lib.m2_mlp_fused_fwd(_ptr(x), _ptr(w_gated), _ptr(w_out), _ptr(bias), _ptr(residual), _ptr(out), M, d, I, nb,
+                               _act_code(out_dtype), _stream()))
+    return out
+
+
 def layernorm(x: Tensor, gamma: Tensor, beta: Tensor, eps: float, want_f32: bool = True, want_bf16: bool = False,
               want_channel_major: bool = False):
     """LayerNorm over the last dim of x (M, d) fp32 -> (f32 (M,d) | None, bf16 (M,d) | None, f32 (d,M) | None)."""

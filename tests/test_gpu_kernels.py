@@ -205,6 +205,13 @@ def test_encoder_small(gpu, L, B, layers):
     out1, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
     e, e2 = rel_err(out1, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
+    # the whole MLP as one kernel (an option as well)
+    for layer in model.encoder.layer:
+        layer.mlp.fuse_wo_layernorm = False
+        layer.mlp.fuse_mlp = True
+    out2, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
+    e, e2 = rel_err(out2, ref)
+    assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
 
 
 def test_encoder_hip_graph_replays_match_eager(gpu):
@@ -591,3 +598,37 @@ def test_bench_prints_its_json_line(gpu, extra):
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=60, cwd=root)
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
+@pytest.mark.parametrize("M,I", [(1, 3072), (100, 3072), (128, 3072), (300, 1536), (4096, 3072), (32768 - 70, 3072),
+                                 (130, 256)])
+def test_mlp_fused_matches_oracle_and_the_two_kernel_path(gpu, M, I):
+    """gated_layers -> GLU -> wo + bias + residual as one kernel (d = 768) against fp64 on the bf16-rounded operands
+    (the gated values rounded to bf16 between the two products, as the two-kernel path and the reference's autocast
+    do), ragged M, both output dtypes, and against m2_blockdiag_glu_fwd + m2_blockdiag_linear_fwd."""
+    from m2_amd import ops
+    from oracle import m2_oracle as O
+    d, nb = 768, 4
+    assert ops.mlp_fused_supported(d, I, nb) and not ops.mlp_fused_supported(1536, 6144, nb)
+    g = torch.Generator().manual_seed(M + I)
+    x = torch.randn(M, d, generator=g).bfloat16()
+    wg = (torch.randn(nb, 2 * I // nb, d // nb, generator=g) * 0.07).bfloat16()
+    wo = (torch.randn(nb, d // nb, I // nb, generator=g) * 0.05).bfloat16()
+    bias = torch.randn(d, generator=g)
+    got = ops.mlp_fused(x.to(gpu), wg.to(gpu), wo.to(gpu), bias.to(gpu), x.to(gpu), out_dtype=torch.float32)
+    h = O.blockdiag_multiply(x.float(), wg.float()).double()
+    a = (torch.nn.functional.gelu(h[:, :I]) * h[:, I:])
+    ref = O.blockdiag_multiply(a.float(), wo.float()).double() + bias.double() + x.double()
+    e, e2 = rel_err(got, ref)
+    assert e < 5e-3 and e2 < 3e-3, (e, e2)          # the only rounding inside is that of the gated values to bf16
+    # the two-kernel path rounds at the same place: agreement to accumulation order
+    g2 = ops.blockdiag_glu(x.to(gpu), wg.to(gpu))
+    two = ops.blockdiag_linear(g2, wo.to(gpu), bias.to(gpu), x.to(gpu), out_dtype=torch.float32)
+    assert rel_err(got, two)[0] < 1e-3
+    got16 = ops.mlp_fused(x.to(gpu), wg.to(gpu), wo.to(gpu), None, None, out_dtype=torch.bfloat16)
+    ref16 = O.blockdiag_multiply(a.float(), wo.float()).double()
+    assert rel_err(got16.float(), ref16)[0] < TOL_BF16
+    with pytest.raises(RuntimeError, match="768"):
+        ops.mlp_fused(torch.zeros(8, 512, device=gpu, dtype=torch.bfloat16),
+                      torch.zeros(4, 256, 128, device=gpu, dtype=torch.bfloat16),
+                      torch.zeros(4, 128, 128, device=gpu, dtype=torch.bfloat16))
