@@ -152,6 +152,33 @@ def cpu_baseline(sd, cfg, ids, mask, B):
                            f"(min {times[0]:.2f}, max {times[2]:.2f})"}
 
 
+def probe_matrix_pipe(iters: int = 4000):
+    """Sustained bf16 MFMA rate of the chip (m2_probe_mfma_fwd) alone and with the company real kernels give it."""
+    import ctypes
+    from m2_amd._lib import check, lib
+    sink = torch.empty(512 * 1024, device="cuda:0")
+    rows = []
+    for reads, valu in ((0, 0), (1, 0), (2, 0), (1, 4), (1, 6), (1, 11)):
+        for wps in (1, 2):
+            n, waves = ctypes.c_longlong(0), ctypes.c_int(0)
+            call = lambda it: check(lib.m2_probe_mfma_fwd(reads, valu, wps, it, ctypes.c_void_p(sink.data_ptr()),
+                                                          ctypes.byref(n), ctypes.byref(waves),
+                                                          torch.cuda.current_stream().cuda_stream))
+            call(10)
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            call(iters)
+            e.record()
+            torch.cuda.synchronize()
+            ms = s.elapsed_time(e)
+            tflops = n.value * waves.value * 32768 / (ms * 1e-3) / 1e12
+            rows.append({"lds_reads_per_mfma": reads, "valu_per_mfma": valu, "waves_per_simd": wps, "ms": ms,
+                         "tflops": tflops, "frac_of_published_peak": tflops / MFMA_BF16_PEAK_TFLOPS})
+    return {"probe": "v_mfma_f32_32x32x16_bf16 loop on all compute units", "published_peak_tflops": MFMA_BF16_PEAK_TFLOPS,
+            "rows": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -168,6 +195,9 @@ def main():
                          "sit inside a graph, so the same K steps run eagerly first, with HIP events around "
                          "every launch, for the roofline object and eager_ms_per_step")
     ap.set_defaults(hip_graph=True)
+    ap.add_argument("--probe", action="store_true",
+                    help="only measure what the matrix pipe sustains on this chip (MFMA loop alone, with LDS operand "
+                         "reads, with vector-ALU work beside it) and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device copy three times (known-size kernel for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -192,6 +222,10 @@ def main():
     import m2_amd
     from m2_amd import ops
 
+    if args.probe:
+        print(json.dumps(probe_matrix_pipe()))
+        return
+
     cfg, B, L, ids, mask, label, idx = workload(args.config)
     d = cfg.hidden_size
     sd = m2_amd.seeded_state_dict(cfg, 1234 + idx)
@@ -210,6 +244,7 @@ def main():
                     ("layernorm", "layernorm"), ("embed_layernorm", "embed_layernorm")):
         wrapped[fn] = timer.wrap(ops, fn, tag)
 
+    model.encoder.overlap_filters = False      # per-kernel timings: filter generation in line, nothing else on the chip
     with torch.no_grad():
         for _ in range(args.warmup):
             out, _ = model(ids_g, attention_mask=mask_g)
@@ -235,6 +270,7 @@ def main():
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 
+    model.encoder.overlap_filters = None       # the default: filter generation of all layers on a second stream
     if args.hip_graph:
         model.encoder.use_hip_graph = True
     with torch.no_grad():
@@ -305,7 +341,7 @@ def main():
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 GEMM / f32 FFT", "data": "synthetic token ids, seeded N(0,0.02) weights",
         "config": {"workload": label, "batch": B, "seq_len": L, "d_model": d, "layers": cfg.num_hidden_layers,
-                   "filters": "regenerated from weights every forward",
+                   "filters": "regenerated from weights every forward, on a second stream beside the layers",
                    "launch": "one captured HIP graph per forward" if args.hip_graph else "eager launches",
                    "eager_ms_per_step": eager_ms,
                    "ms_per_step_with_cached_filter_spectra": cached_ms},

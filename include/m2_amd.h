@@ -131,6 +131,16 @@ int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, const float* u,
 int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, int L, int d, int act_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Dense projection of the sequence mixer (in_linear, bert/src/mm/monarch_mixer_sequence_mixer.py:81,108) written
+ * straight into the channel-major layout m2_mixer_core_fwd reads:
+ *   out[q][p] = sum_k Q[q][k] P[p][k],   P (np, K), Q (nq, K), out (nq, np), all bf16, dense, fp32 accumulation.
+ * With P = the layer input (M, d) and Q = in_linear.weight (3d, d) the result is xproj (3d, M); the bias is left
+ * to m2_mixer_core_fwd (proj_bias).  The reference runs this as nn.Linear followed by a transpose.
+ * Needs K % 64 == 0 and operands below 4 GiB each. */
+int m2_gemm_bf16_supported(int np, int nq, int K);
+int m2_gemm_bf16_qmajor_fwd(const void* P, const void* Q, void* out, int np, int nq, int K, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Block-diagonal ("Monarch") linear layers of the GLU MLP, bf16 MFMA with fp32 accumulation.
  * Stand in for: bert/src/mm/blockdiag_multiply.py:49-60 (BlockdiagMultiply.forward, bf16 under
  * autocast), bert/src/mm/structured_linear.py:65-69 (bias add) and bert/src/bert_layers.py:482-506
@@ -150,6 +160,14 @@ int m2_blockdiag_glu_fwd(const void* x, const void* w, void* out, int M, int in_
  * Needs (in/nblocks) % 64 == 0, (out/nblocks) % 64 == 0. */
 int m2_blockdiag_linear_fwd(const void* x, const void* w, const float* bias, const void* residual, void* out, int M,
                             int in_features, int out_features, int nblocks, int out_dtype, void* stream);
+
+/* The fp32 form: out = blockdiag_multiply(x, w) (+ bias) with fp32 operands, exact fp32 products and fp32
+ * accumulation -- what the reference computes when BlockdiagLinear is called with fp32 tensors outside CUDA autocast
+ * (bert/src/mm/blockdiag_multiply.py:50 casts to bf16 only under autocast).  x (M, in_features) fp32; w (nblocks,
+ * out/nblocks, in/nblocks) fp32; bias (out_features) fp32 or NULL; out (M, out_features) fp32.
+ * Needs (in_features / nblocks) % 8 == 0. */
+int m2_blockdiag_linear_f32_fwd(const float* x, const float* w, const float* bias, float* out, int M, int in_features,
+                                int out_features, int nblocks, void* stream);
 
 /* The whole GLU MLP up to the LayerNorm input in one kernel, the (M, 2I) and (M, I) intermediates never leaving the
  * chip:  out = blockdiag_multiply(gelu_erf(h[:, :I]) * h[:, I:], w_out) (+ bias) (+ residual),
@@ -198,6 +216,17 @@ int m2_embed_layernorm_fwd(const long long* input_ids, const long long* token_ty
                            int type_vocab_size, int max_positions, const float* gamma, const float* beta, float eps,
                            float* out_f32, void* out_bf16, float* out_channel_major, int* bad_index, int B, int L,
                            int d, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Measurement aid (no counterpart in the reference): a loop of 12 * iters v_mfma_f32_32x32x16_bf16 per wave on every
+ * compute unit, alone or accompanied by 1 or 2 software-pipelined 16-byte LDS operand reads per MFMA and by 0, 4, 6
+ * or 11 fp32 FMAs per MFMA in the same wave, at 1 or 2 waves per SIMD.  The caller times the stream around the call;
+ * 32768 flop per MFMA, *mfma_per_wave MFMAs in each of *waves waves.  bench.py --probe prints the rates: they are the
+ * ceilings the GEMM-shaped kernels are held against beside the published peak.  sink: device buffer of at least
+ * 512 floats per compute unit (written so that the loop is not optimised away).
+ * Supported (lds_reads_per_mfma, valu_per_mfma): (0,0) (1,0) (2,0) (1,4) (1,6) (1,11). */
+int m2_probe_mfma_fwd(int lds_reads_per_mfma, int valu_per_mfma, int waves_per_simd, int iters, float* sink,
+                      long long* mfma_per_wave, int* waves, void* stream);
 
 #ifdef __cplusplus
 }

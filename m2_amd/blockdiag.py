@@ -1,10 +1,11 @@
 """BlockdiagLinear / blockdiag_multiply with the reference's interface, on bf16 MFMA.
 
 Reference: bert/src/mm/blockdiag_linear.py:12-48, bert/src/mm/structured_linear.py:11-69,
-bert/src/mm/blockdiag_multiply.py:19-60.  The arithmetic is always bf16 x bf16 with fp32
-accumulation (what the reference does under CUDA autocast); the result comes back in the input's
-dtype.  Inputs are zero-padded to `in_features_extended` and outputs cropped to `out_features` like
-the reference's preprocess / postprocess.
+bert/src/mm/blockdiag_multiply.py:19-60.  Under CUDA autocast, or with bf16 input, the arithmetic is
+bf16 x bf16 with fp32 accumulation and a bf16 result (the reference's `custom_fwd(cast_inputs=bf16)`);
+with fp32 input outside autocast it is fp32 throughout, as in the reference.  Inputs are zero-padded
+to `in_features_extended` and outputs cropped to `out_features` like the reference's preprocess /
+postprocess.
 """
 from __future__ import annotations
 
@@ -17,6 +18,11 @@ import torch.nn.functional as F
 from . import ops
 
 
+def _fp32_path(x: torch.Tensor) -> bool:
+    """fp32 arithmetic exactly when the reference would use it: fp32 input and no CUDA autocast."""
+    return x.dtype == torch.float32 and not torch.is_autocast_enabled()
+
+
 def blockdiag_multiply(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """x (..., nblocks*p), weight (nblocks, q, p) -> (..., nblocks*q)."""
     if not x.is_cuda:
@@ -24,6 +30,9 @@ def blockdiag_multiply(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     nb, q, p = weight.shape
     if x.shape[-1] != nb * p:
         raise ValueError(f"last dim {x.shape[-1]} != nblocks*p = {nb * p}")
+    if _fp32_path(x) and p % 8 == 0:
+        out = ops.blockdiag_linear_f32(x.reshape(-1, nb * p).contiguous(), weight.detach().float().contiguous())
+        return out.view(*x.shape[:-1], nb * q)
     x2 = x.reshape(-1, nb * p).to(torch.bfloat16).contiguous()
     w = weight.detach().to(torch.bfloat16).contiguous()
     out_dtype = torch.bfloat16 if (x.dtype == torch.bfloat16 or torch.is_autocast_enabled()) else torch.float32
@@ -80,15 +89,20 @@ class BlockdiagLinear(nn.Module):
             raise RuntimeError("BlockdiagLinear (m2_amd) runs on the GPU only")
         if x.shape[-1] < self.in_features_extended:
             x = F.pad(x, (0, self.in_features_extended - x.shape[-1]))
-        x2 = x.reshape(-1, self.in_features_extended).to(torch.bfloat16).contiguous()
-        out_dtype = torch.bfloat16 if (x.dtype == torch.bfloat16 or torch.is_autocast_enabled()) else torch.float32
         bias = None
         if self.bias is not None:
             bias = self.bias.detach().float()
             if self.out_features_extended > self.out_features:
                 bias = F.pad(bias, (0, self.out_features_extended - self.out_features))
             bias = bias.contiguous()
-        out = ops.blockdiag_linear(x2, self.weight_bf16(), bias, None, out_dtype=out_dtype)
+        nb, q, p = self.weight.shape
+        if _fp32_path(x) and p % 8 == 0:
+            out = ops.blockdiag_linear_f32(x.reshape(-1, self.in_features_extended).contiguous(),
+                                           self.weight.detach().float().contiguous(), bias)
+        else:
+            x2 = x.reshape(-1, self.in_features_extended).to(torch.bfloat16).contiguous()
+            out_dtype = torch.bfloat16 if (x.dtype == torch.bfloat16 or torch.is_autocast_enabled()) else torch.float32
+            out = ops.blockdiag_linear(x2, self.weight_bf16(), bias, None, out_dtype=out_dtype)
         out = out.view(*x.shape[:-1], self.out_features_extended)
         if self.out_features_extended > self.out_features:
             out = out[..., :self.out_features]

@@ -858,6 +858,51 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
   store_tile((nslab - 1) & 1, m_begin + 32 * (nslab - 1));
 }
 
+// ---------------------------------------------------------------------------------------------
+// fp32 block-diagonal multiply: what the reference computes when it is called with fp32 tensors outside CUDA autocast
+// (bert/src/mm/blockdiag_multiply.py:50 casts to bf16 only under autocast).  v_mfma_f32_32x32x2_f32 (exact fp32
+// products, fp32 accumulation); a wave owns a 32 x 32 output tile and reads both operands straight from global
+// memory in operand layout: lane (i, h) takes 4 consecutive K values of x row i and of weight row i per step, which
+// feed four MFMAs (MFMA j of a step contracts K = 8 s + j from the lanes h = 0 and K = 8 s + 4 + j from h = 1).
+// Not a hot path of the encoder (that runs under autocast): no LDS tiling.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void blockdiag_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                            const float* __restrict__ bias, float* __restrict__ out,
+                                                            int M, int nb, int p, int q) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i32 = lane & 31, half = lane >> 5;
+  const int tiles_n = (q + 31) / 32;                       // column tiles per block
+  const int tile = blockIdx.x * 4 + wave;                  // over (row tile, block, column tile)
+  const int ntiles = ((M + 31) / 32) * nb * tiles_n;
+  if (tile >= ntiles) return;
+  const int tn = tile % tiles_n, blk = (tile / tiles_n) % nb, tm = tile / (tiles_n * nb);
+  int row = tm * 32 + i32, col = tn * 32 + i32;
+  const bool col_ok = col < q;
+  row = row < M ? row : M - 1;
+  col = col_ok ? col : q - 1;
+  const float* xr = x + (long)row * nb * p + (long)blk * p + 4 * half;
+  const float* wr = w + ((long)blk * q + col) * p + 4 * half;
+  floatx16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  for (int k = 0; k < p; k += 8) {
+    const float4 a = *reinterpret_cast<const float4*>(xr + k);
+    const float4 b = *reinterpret_cast<const float4*>(wr + k);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc, 0, 0, 0);
+  }
+  // accumulator element v: x row 8 (v / 4) + 4 half + v % 4 of the tile, output column i32
+  if (!col_ok) return;
+  const int oc = blk * q + tn * 32 + i32;
+  const float bv = bias ? bias[oc] : 0.f;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int r = tm * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+    if (r < M) out[(long)r * nb * q + oc] = acc[v] + bv;
+  }
+}
+
 template <int KS>
 static int launch_glu_ws(const void* x, const void* w, void* out, int M, int nb, int q, hipStream_t stream) {
   constexpr int p = 16 * KS;
@@ -951,6 +996,21 @@ extern "C" int m2_blockdiag_linear_fwd(const void* x, const void* w, const float
                 : launch_blockdiag<4, 1, false, float, 1>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st);
   return wide ? launch_blockdiag<2, 2, false, uint16_t, 1>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st)
               : launch_blockdiag<4, 1, false, uint16_t, 1>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st);
+}
+
+extern "C" int m2_blockdiag_linear_f32_fwd(const float* x, const float* w, const float* bias, float* out, int M,
+                                           int in_features, int out_features, int nblocks, void* stream) {
+  if (!x || !w || !out) return set_error(M2_ERR_ARG, "m2_blockdiag_linear_f32_fwd: null pointer");
+  if (M <= 0 || nblocks <= 0 || in_features <= 0 || out_features <= 0 || in_features % nblocks || out_features % nblocks)
+    return set_error(M2_ERR_UNSUPPORTED, "m2_blockdiag_linear_f32_fwd: in=%d and out=%d must be positive multiples of nblocks=%d",
+                     in_features, out_features, nblocks);
+  const int p = in_features / nblocks, q = out_features / nblocks;
+  if (p % 8 != 0) return set_error(M2_ERR_UNSUPPORTED, "m2_blockdiag_linear_f32_fwd: in_features/nblocks=%d must be a multiple of 8", p);
+  const long ntiles = (long)((M + 31) / 32) * nblocks * ((q + 31) / 32);
+  if ((ntiles + 3) / 4 > 0x7fffffffL) return set_error(M2_ERR_UNSUPPORTED, "m2_blockdiag_linear_f32_fwd: too many tiles");
+  hipLaunchKernelGGL(blockdiag_f32_kernel, dim3((unsigned)((ntiles + 3) / 4)), dim3(256), 0, (hipStream_t)stream, x, w, bias,
+                     out, M, nblocks, p, q);
+  return check_launch("blockdiag_f32");
 }
 
 template <bool EMBED>

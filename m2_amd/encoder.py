@@ -212,7 +212,10 @@ class BertLayer(nn.Module):
         # output: the same product as W @ h16^T, for which the library picks a faster kernel (126 against 144 us at
         # M = 32768, d = 768)
         xproj = torch.empty(3 * d, B * L, dtype=torch.bfloat16, device=h16.device)
-        torch.mm(h16, w_in.t(), out=xproj.t())
+        if at.own_in_linear:
+            ops.gemm_qmajor(h16, w_in, out=xproj)
+        else:
+            torch.mm(h16, w_in.t(), out=xproj.t())
         if spec_ready is not None:
             torch.cuda.current_stream().wait_event(spec_ready)
         y = at.core(xproj.view(3 * d, B, L), hT.view(d, B, L) if at.residual_long_conv else None, B, L, spec=spec)
@@ -231,7 +234,7 @@ class BertEncoder(nn.Module):
     it), `.to()` / `.cuda()` and `reset_graphs()`; call `reset_graphs()` after changing a parameter in place.
     Nothing in the captured region uses a memset."""
 
-    OVERLAP_UPFRONT_MAX_L = 2048
+    UPFRONT_MAX_BYTES = 16 << 30
 
     def __init__(self, config: M2BertConfig, use_hip_graph: bool = False):
         super().__init__()
@@ -245,10 +248,10 @@ class BertEncoder(nn.Module):
         #              for its own (holds all spectra at once: 100 MB per layer at L = 8192, d = 768);
         #   True       the spectra of layer i + 1 behind the mixer core of layer i;
         #   False      in line, on the main stream;
-        #   None       "upfront" for sequences up to OVERLAP_UPFRONT_MAX_L, where the generation kernels are a few
-        #              workgroups each and pure latency (forward as one HIP graph at d = 768: -10 % at L = 256,
-        #              -7 % at L = 1024, -2 % at L = 2048 .. 8192), in line beyond, where concurrent kernels also
-        #              blur per-kernel timings.
+        #   None       "upfront" while all layers' spectra together stay below UPFRONT_MAX_BYTES, else True.
+        # Measured on MI355X, forward as one HIP graph, in line / "upfront" / True: 8.71 / 8.45 / 8.64 ms at
+        # L = 8192, B = 4; 15.22 / 14.54 / 14.89 ms at L = 32768, B = 1; 11.00 / 10.47 / 10.75 ms for 24 x 1536 at
+        # L = 128, B = 64.  Kernels of the two streams then share the chip, so per-kernel timings are taken in line.
         self.overlap_filters = None
         self._filter_stream = None
         # nn.Module.load_state_dict of a parent never calls a child's load_state_dict, but it does run the
@@ -286,7 +289,9 @@ class BertEncoder(nn.Module):
             cur = torch.cuda.current_stream()
             overlap = self.overlap_filters
             if overlap is None:
-                overlap = "upfront" if L <= self.OVERLAP_UPFRONT_MAX_L else False
+                d = self.layer[0].attention.d_model
+                total = len(self.layer) * ops.lib.m2_filter_spectrum_bytes(d, L)
+                overlap = "upfront" if total <= self.UPFRONT_MAX_BYTES else True
             nxt = [None, None]                       # spectra of the next layer and the event that says they are ready
             if overlap:
                 if self._filter_stream is None:

@@ -3,8 +3,10 @@ arithmetic done by the HIP kernels of libm2_amd.so.
 
 Reference: bert/src/mm/hyena_utils.py:50-63 (Sin), :66-88 (PositionalEmbedding), :91-112
 (ExponentialModulation), :115-248 (HyenaFilter), bert/src/utils/train.py:4-17 (OptimModule).
-The submodules hold parameters and buffers under the same names; their own `forward`s are not
-part of the GPU path (the whole filter is produced by `m2_hyena_filter_fwd`) and raise if called.
+The submodules hold parameters and buffers under the same names.  The hot path does not call their
+`forward`s (the whole filter is produced by `m2_hyena_filter_fwd`); a caller that evaluates them directly, as
+bert/src/mm/flash_mm.py:141-149 does with `filter_fn.implicit_filter(z)`, gets the reference's own expressions
+as plain torch ops on whatever device the tensors live on.
 """
 from __future__ import annotations
 
@@ -35,18 +37,18 @@ class OptimModule(nn.Module):
             setattr(getattr(self, name), "_optim", optim)
 
 
-class _KernelEvaluated(nn.Module):
-    def forward(self, *args, **kwargs):
-        raise NotImplementedError(
-            f"{type(self).__name__} is evaluated inside the fused HyenaFilter kernel; call HyenaFilter.filter()")
+class Sin(nn.Module):
+    """sin(w_mod * freq * x) (bert/src/mm/hyena_utils.py:50-63); one instance, hence one `freq`, is shared by every
+    activation slot of both implicit-filter MLPs."""
 
-
-class Sin(_KernelEvaluated):
     def __init__(self, dim, w=10, w_mod=1, train_freq=True):
         super().__init__()
         init = w * torch.ones(1, dim)
         self.freq = nn.Parameter(init) if train_freq else init
         self.w_mod = w_mod
+
+    def forward(self, x):
+        return torch.sin(self.w_mod * self.freq * x)
 
 
 class PositionalEmbedding(OptimModule):
@@ -61,19 +63,17 @@ class PositionalEmbedding(OptimModule):
         return self.z[:, :L], self.t[:, :L]
 
 
-class ExponentialModulation(OptimModule, _KernelEvaluated):
+class ExponentialModulation(OptimModule):
     def __init__(self, d_model, fast_decay_pct=0.3, slow_decay_pct=1.5, target=1e-2, modulation_lr=0.0,
                  shift: float = 0.0, **kwargs):
         super().__init__()
         self.shift = shift
         self.register("deltas", modulation_deltas(d_model, fast_decay_pct, slow_decay_pct, target), lr=modulation_lr)
 
-
-class _HeldLinear(nn.Linear):
-    """nn.Linear used as a parameter holder inside the implicit-filter Sequential."""
-
-    def forward(self, x):
-        raise NotImplementedError("implicit-filter layers are evaluated inside the fused HyenaFilter kernel")
+    def forward(self, t, x):
+        """x * (exp(-t |deltas|) + shift) (bert/src/mm/hyena_utils.py:110-112)."""
+        decay = torch.exp(-t * self.deltas.abs())
+        return x * (decay + self.shift)
 
 
 class HyenaFilter(OptimModule):
@@ -103,8 +103,8 @@ class HyenaFilter(OptimModule):
         self.pos_emb = PositionalEmbedding(emb_dim, seq_len, lr_pos_emb)
 
         def mlp():
-            return nn.Sequential(_HeldLinear(emb_dim, order), act, _HeldLinear(order, order), act,
-                                 _HeldLinear(order, order), act, _HeldLinear(order, d_model, bias=False))
+            return nn.Sequential(nn.Linear(emb_dim, order), act, nn.Linear(order, order), act,
+                                 nn.Linear(order, order), act, nn.Linear(order, d_model, bias=False))
 
         self.implicit_filter = mlp()
         if self.bidirectional:

@@ -152,6 +152,23 @@ def fftconv(x: Tensor, spec: Tensor, B: int, L: int, d: int) -> Tensor:
     return out
 
 
+def gemm_qmajor(P: Tensor, Q: Tensor, out: Optional[Tensor] = None) -> Tensor:
+    """out (nq, np) = Q @ P^T for P (np, K), Q (nq, K) bf16 (fp32 accumulation): with P the tokens (M, d) and Q a
+    weight (n, d) this is the projection written channel-major (n, M)."""
+    np_, K = P.shape
+    nq, K2 = Q.shape
+    _require(P, "P", torch.bfloat16)
+    _require(Q, "Q", torch.bfloat16)
+    if K != K2:
+        raise ValueError(f"P has K = {K}, Q has K = {K2}")
+    if out is None:
+        out = torch.empty(nq, np_, dtype=torch.bfloat16, device=P.device)
+    else:
+        _require(out, "out", torch.bfloat16, (nq, np_))
+    check(lib.m2_gemm_bf16_qmajor_fwd(_ptr(P), _ptr(Q), _ptr(out), np_, nq, K, _stream()))
+    return out
+
+
 def blockdiag_glu(x: Tensor, w: Tensor, out: Optional[Tensor] = None) -> Tensor:
     """gelu_erf(h[:, :I]) * h[:, I:] with h = blockdiag_multiply(x, w); x (M, in) bf16, w (nb, 2I/nb, in/nb) bf16."""
     M, in_f = x.shape
@@ -189,6 +206,22 @@ def blockdiag_linear(x: Tensor, w: Tensor, bias: Optional[Tensor] = None, residu
         _require(out, "out", out_dtype, (M, out_f))
     check(lib.m2_blockdiag_linear_fwd(_ptr(x), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out), M, in_f, out_f, nb,
                                       _act_code(out_dtype), _stream()))
+    return out
+
+
+def blockdiag_linear_f32(x: Tensor, w: Tensor, bias: Optional[Tensor] = None) -> Tensor:
+    """blockdiag_multiply(x, w) (+ bias) in fp32 (exact fp32 products, fp32 accumulation); x (M, in) fp32,
+    w (nb, out/nb, in/nb) fp32."""
+    M, in_f = x.shape
+    nb, q, p = w.shape
+    _require(x, "x", torch.float32)
+    _require(w, "w", torch.float32)
+    if nb * p != in_f:
+        raise ValueError(f"x has {in_f} features, weight expects {nb}*{p}")
+    if bias is not None:
+        _require(bias, "bias", torch.float32, (nb * q,))
+    out = torch.empty(M, nb * q, dtype=torch.float32, device=x.device)
+    check(lib.m2_blockdiag_linear_f32_fwd(_ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, in_f, nb * q, nb, _stream()))
     return out
 
 

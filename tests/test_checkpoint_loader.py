@@ -88,3 +88,57 @@ def test_context_extension_128_to_512(tile_z):
         assert p + "pos_emb.z" in missing
     assert torch.equal(got[p + "implicit_filter.0.weight"], sd[p + "implicit_filter.0.weight"])
     assert "embeddings.position_ids" in missing and p + "pos_emb.t" in missing
+
+
+def test_context_extension_reference_mode_writes_the_old_table_into_slots_of_a_zero_tensor():
+    """mode="reference": `z_new = zeros(new_len); for k in range(2, R): z_new[(k-1) L_old : k L_old] = z_old`
+    (bert/src/bert_layers.py:1141-1151) -- slot 0 stays zero, slots 1 .. R - 2 hold copies, the rest stays zero.
+    Built here from that formula for the reference's own cases 8192 -> 32768 (R = 5) and 128 -> 2048 (R = 17),
+    and for a length the reference has no entry for (every slot but the first)."""
+    for old, new, R in ((8192, 32768, 5), (128, 2048, 17), (128, 1024, 17), (256, 1024, None)):
+        z_old = torch.randn(1, old, 5, generator=torch.Generator().manual_seed(old))
+        sd = {"encoder.layer.0.attention.filter_fn.pos_emb.z": z_old,
+              "encoder.layer.0.attention.filter_fn.pos_emb.t": torch.zeros(1, old, 1),
+              "embeddings.position_embeddings.weight": torch.randn(old, 8),
+              "embeddings.position_ids": torch.arange(old)[None]}
+        out = m2_amd.extend_context(sd, new, mode="reference")
+        want = torch.zeros(1, new, 5)
+        ks = range(2, R) if R is not None else range(2, new // old + 1)
+        for k in ks:
+            if k * old <= new:
+                want[:, (k - 1) * old:k * old, :] = z_old
+        got = out["encoder.layer.0.attention.filter_fn.pos_emb.z"]
+        assert torch.equal(got, want), (old, new)
+        assert not got[:, :old].any() and torch.equal(got[:, old:2 * old], z_old)
+        assert "encoder.layer.0.attention.filter_fn.pos_emb.t" not in out and "embeddings.position_ids" not in out
+        assert out["embeddings.position_embeddings.weight"].shape[0] == new
+    with pytest.raises(ValueError, match="unknown"):
+        m2_amd.extend_context(sd, 1024, mode="zeros")
+    # through the loader: the model's z becomes the zero-slotted table
+    short = m2_amd.m2_bert_80m(128)
+    short.num_hidden_layers = 1
+    long = m2_amd.m2_bert_80m(512)
+    long.num_hidden_layers = 1
+    sd = m2_amd.seeded_state_dict(short, 29)
+    model = m2_amd.BertModel(long)
+    m2_amd.load_reference_checkpoint(model, sd, extend_to=512, z_mode="reference", max_missing=16)
+    z = model.state_dict()["encoder.layer.0.attention.filter_fn2.pos_emb.z"]
+    zo = sd["encoder.layer.0.attention.filter_fn2.pos_emb.z"]
+    assert not z[:, :128].any() and all(torch.equal(z[:, 128 * s:128 * (s + 1)], zo) for s in (1, 2, 3))
+
+
+def test_filter_submodules_compute_the_reference_expressions():
+    """Sin, ExponentialModulation and the implicit-filter Sequential evaluate on their own (plain torch ops), so that a
+    caller doing `filter_fn.implicit_filter(z)` and `filter_fn.modulation(t, h)` gets the filter the kernel produces."""
+    from oracle import m2_oracle as O
+    cfg = m2_amd.m2_bert_80m(64)
+    cfg.hidden_size = 64
+    sd = m2_amd.seeded_state_dict(cfg, 3, std=0.2, what="mixer")
+    fn = m2_amd.HyenaFilter(64, emb_dim=5, order=128, seq_len=64, bidirectional=True, w=10)
+    fn.load_state_dict({k[len("filter_fn."):]: v for k, v in sd.items() if k.startswith("filter_fn.")})
+    z, t = fn.pos_emb(64)
+    h = fn.modulation(t, fn.implicit_filter(z))
+    hr = fn.modulation(t, fn.implicit_filter_rev(z))
+    assert torch.allclose(h, O.hyena_filter_taps(sd, "filter_fn.", 64, rev=False), atol=1e-6)
+    assert torch.allclose(hr, O.hyena_filter_taps(sd, "filter_fn.", 64, rev=True), atol=1e-6)
+    assert fn.implicit_filter[1] is fn.implicit_filter[3] is fn.implicit_filter_rev[5]      # one shared Sin

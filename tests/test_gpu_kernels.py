@@ -205,10 +205,11 @@ def test_encoder_small(gpu, L, B, layers):
     out1, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
     e, e2 = rel_err(out1, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
-    # the whole MLP as one kernel (an option as well)
+    # the whole MLP as one kernel, and the in-projection on this library's own GEMM kernel (options as well)
     for layer in model.encoder.layer:
         layer.mlp.fuse_wo_layernorm = False
         layer.mlp.fuse_mlp = True
+        layer.attention.own_in_linear = True
     out2, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
     e, e2 = rel_err(out2, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
@@ -632,3 +633,49 @@ def test_mlp_fused_matches_oracle_and_the_two_kernel_path(gpu, M, I):
         ops.mlp_fused(torch.zeros(8, 512, device=gpu, dtype=torch.bfloat16),
                       torch.zeros(4, 256, 128, device=gpu, dtype=torch.bfloat16),
                       torch.zeros(4, 128, 128, device=gpu, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("np_,nq,K", [(256, 256, 64), (4096, 2304, 768), (1000, 300, 128), (32768, 2304, 768),
+                                     (8192, 4608, 1536), (257, 513, 192)])
+def test_gemm_qmajor_projection(gpu, np_, nq, K):
+    """The dense projection kernel (in_linear written channel-major) against fp64 on the bf16 operands, ragged
+    tiles both ways."""
+    from m2_amd import ops
+    g = torch.Generator().manual_seed(np_ + nq)
+    P = torch.randn(np_, K, generator=g).bfloat16()
+    Q = (torch.randn(nq, K, generator=g) * 0.05).bfloat16()
+    got = ops.gemm_qmajor(P.to(gpu), Q.to(gpu))
+    assert got.shape == (nq, np_) and got.dtype == torch.bfloat16
+    ref = (Q.float() @ P.float().T).double() if np_ * nq > 4e6 else Q.double() @ P.double().T
+    e, e2 = rel_err(got.float(), ref)
+    assert e < TOL_BF16 and e2 < 4e-3, (e, e2)
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        ops.gemm_qmajor(torch.zeros(8, 100, device=gpu, dtype=torch.bfloat16), torch.zeros(8, 100, device=gpu, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("M,in_f,out_f,nb", [(300, 768, 6144, 4), (65, 256, 100, 4), (1, 64, 8, 2), (1000, 3072, 768, 4)])
+def test_blockdiag_linear_fp32_outside_autocast(gpu, M, in_f, out_f, nb):
+    """BlockdiagLinear / blockdiag_multiply with fp32 input and no autocast compute in fp32 (1e-4 against fp64), as
+    the reference does on that call; under autocast the same module rounds its operands to bf16."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    g = torch.Generator().manual_seed(M + out_f)
+    lin = m2_amd.BlockdiagLinear(in_f, out_f, bias=True, nblocks=nb)
+    with torch.no_grad():
+        lin.weight.copy_(torch.randn(lin.weight.shape, generator=g) * 0.05)
+        lin.bias.copy_(torch.randn(out_f, generator=g))
+    x = torch.randn(2, M, in_f, generator=g)
+    ref = O.blockdiag_linear(x.double(), lin.weight.detach().double(), lin.bias.detach().double(), in_f, out_f)
+    lin = lin.to(gpu)
+    got = lin(x.to(gpu))
+    assert got.dtype == torch.float32 and got.shape == (2, M, out_f)
+    e, e2 = rel_err(got, ref)
+    assert e < 2e-6 and e2 < 2e-6, (e, e2)
+    got_mul = m2_amd.blockdiag_multiply(x.to(gpu), lin.weight)
+    assert rel_err(got_mul, O.blockdiag_multiply(x.double(), lin.weight.detach().double().cpu()))[0] < 2e-6
+    if (in_f // nb) % 64 == 0 and (out_f // nb) % 64 == 0:
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            low = lin(x.to(gpu))
+        assert low.dtype == torch.bfloat16
+        e = rel_err(low.float(), ref)[0]
+        assert 1e-4 < e < TOL_BF16, e
