@@ -31,23 +31,22 @@ __device__ __forceinline__ bf16x8 ld8(const uint16_t* p) {
   return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
 
-// x * Phi(x), Phi(x) - 1/2 = erf(x / sqrt2) / 2 as an odd polynomial of degree 17 on |x| <= 4.2 (clamped
-// beyond, where Phi is within 1.4e-5 of 0 or 1).  Least-squares fit on Chebyshev nodes; against the fp64
-// erf form the result is within 7.6e-5 absolute for every fp32 x in [-9, 9] (checked on the CPU) -- a
-// fraction of the bf16 rounding the caller applies -- and it costs 12 VALU instructions and no
-// transcendental, where libm erff cost more vector ALU time than the GEMM cost MFMA time.
+// x * Phi(x), Phi(x) - 1/2 = erf(x / sqrt2) / 2 as an odd polynomial of degree 13 on |x| <= 3.9 (clamped beyond,
+// where Phi is within 5e-5 of 0 or 1).  Least-squares fit on Chebyshev nodes; evaluated in fp32 the result is within
+// 1.8e-4 absolute of the fp64 erf form for every fp32 x in [-9, 9] (checked on the CPU), below the bf16 rounding the
+// caller applies to it wherever the result is larger than 0.05 and a fraction of a per cent of the layer's output
+// scale below that.  10 vector-ALU instructions and no transcendental: the GLU epilogue, not the product, bounds
+// the gated kernel, so two multiply-adds less per output (degree 17 gave 7.6e-5) are worth more than the digits.
 __device__ __forceinline__ float gelu_erf(float x) {
-  const float xc = __builtin_amdgcn_fmed3f(x, -4.2f, 4.2f);
+  const float xc = __builtin_amdgcn_fmed3f(x, -3.9f, 3.9f);
   const float x2 = xc * xc;
-  float p = 5.7684985601e-11f;
-  p = fmaf(p, x2, -5.4613545547e-09f);
-  p = fmaf(p, x2, 2.2906412775e-07f);
-  p = fmaf(p, x2, -5.6740019522e-06f);
-  p = fmaf(p, x2, 9.3766078270e-05f);
-  p = fmaf(p, x2, -1.1098775728e-03f);
-  p = fmaf(p, x2, 9.8181711574e-03f);
-  p = fmaf(p, x2, -6.6345343288e-02f);
-  p = fmaf(p, x2, 3.9890193482e-01f);
+  float p = 2.7693410957e-08f;
+  p = fmaf(p, x2, -1.8473178272e-06f);
+  p = fmaf(p, x2, 5.2869800351e-05f);
+  p = fmaf(p, x2, -8.6171873090e-04f);
+  p = fmaf(p, x2, 9.0065851481e-03f);
+  p = fmaf(p, x2, -6.5103946404e-02f);
+  p = fmaf(p, x2, 3.9828952833e-01f);
   return x * fmaf(p, xc, 0.5f);
 }
 
@@ -825,12 +824,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     product((s + 1) & 1, gb, vb);
     epilogue(s & 1, ga, va);
     // issue order inside this block: one MFMA, its next operand read, then a share of the epilogue's vector ALU
-    // work (about 9 instructions per MFMA) and LDS writes, so that the two pipes run side by side
+    // work (about 8 instructions per MFMA) and LDS writes, so that the two pipes run side by side
     __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);      // operand reads run six MFMAs ahead
     static_for<0, 2 * KS>([&](auto) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, (216 + 2 * KS - 1) / (2 * KS), 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, (184 + 2 * KS - 1) / (2 * KS), 0);
       __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
     });
     if (s + 2 < nslab) {

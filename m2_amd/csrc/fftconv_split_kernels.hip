@@ -107,30 +107,44 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
         b1 = sb[c]; b2 = sb[d + c]; bv = sb[2 * d + c];
         if (pbias) { p1 = pbias[c]; p2 = pbias[d + c]; pv = pbias[2 * d + c]; }
       }
+      // The bias p of the in-projection is not added to the inputs: a 3-tap convolution of (x + p) is the convolution
+      // of x plus p (w0 + w1 + w2), which goes into the convolution's own bias -- except for the first two outputs
+      // of a row, where one or two taps fall on the zero padding (outside the biased signal): those are corrected.
+      const float f1 = b1 + p1 * (w1[0] + w1[1] + w1[2]), f2 = b2 + p2 * (w2[0] + w2[1] + w2[2]),
+                  fv = bv + pv * (wv[0] + wv[1] + wv[2]);
       __builtin_amdgcn_sched_barrier(0);
       static_for<0, 4>([&](auto qq) {
         constexpr int q = decltype(qq)::value;
         const int n = n0 + 8 * q;
         float in[10], a[8], gt[8];
         if constexpr (FULL) {
-          r1.template expand<q>(n, p1, in);
+          float cv[8];
+          r1.template expand<q>(n, in);
           static_for<0, 8>([&](auto ee) {
             constexpr int e = decltype(ee)::value;
-            a[e] = b1 + w1[0] * in[e] + w1[1] * in[e + 1] + w1[2] * in[e + 2];
+            a[e] = f1 + w1[0] * in[e] + w1[1] * in[e + 1] + w1[2] * in[e + 2];
           });
-          rv.template expand<q>(n, pv, in);
+          rv.template expand<q>(n, in);
           static_for<0, 8>([&](auto ee) {
             constexpr int e = decltype(ee)::value;
-            a[e] *= bv + wv[0] * in[e] + wv[1] * in[e + 1] + wv[2] * in[e + 2];
+            cv[e] = fv + wv[0] * in[e] + wv[1] * in[e + 1] + wv[2] * in[e + 2];
           });
-          r2.template expand<q>(n, p2, in);
+          r2.template expand<q>(n, in);
           static_for<0, 8>([&](auto ee) {
             constexpr int e = decltype(ee)::value;
-            gt[e] = b2 + w2[0] * in[e] + w2[1] * in[e + 1] + w2[2] * in[e + 2];
+            gt[e] = f2 + w2[0] * in[e] + w2[1] * in[e + 1] + w2[2] * in[e + 2];
           });
+          if constexpr (q == 0) {
+            if (t == 0) {      // time steps 0 and 1 of the row
+              a[0] -= p1 * (w1[0] + w1[1]); a[1] -= p1 * w1[0];
+              cv[0] -= pv * (wv[0] + wv[1]); cv[1] -= pv * wv[0];
+              gt[0] -= p2 * (w2[0] + w2[1]); gt[1] -= p2 * w2[0];
+            }
+          }
+          static_for<0, 8>([&](auto ee) { a[decltype(ee)::value] *= cv[decltype(ee)::value]; });
         } else {
           // plain long convolution: xproj is a single (d, B, L) signal, no short conv, no gates
-          r1.template expand<q>(n, 0.f, in);
+          r1.template expand<q>(n, in);
           static_for<0, 8>([&](auto ee) {
             constexpr int e = decltype(ee)::value;
             a[e] = in[e + 2];

@@ -45,17 +45,15 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 // x * Phi(x): the same clamped odd polynomial as the separate GLU kernel (blockdiag_kernels.hip), so both paths
 // round alike.
 __device__ __forceinline__ float gelu_erf_poly(float x) {
-  const float xc = __builtin_amdgcn_fmed3f(x, -4.2f, 4.2f);
+  const float xc = __builtin_amdgcn_fmed3f(x, -3.9f, 3.9f);
   const float x2 = xc * xc;
-  float p = 5.7684985601e-11f;
-  p = fmaf(p, x2, -5.4613545547e-09f);
-  p = fmaf(p, x2, 2.2906412775e-07f);
-  p = fmaf(p, x2, -5.6740019522e-06f);
-  p = fmaf(p, x2, 9.3766078270e-05f);
-  p = fmaf(p, x2, -1.1098775728e-03f);
-  p = fmaf(p, x2, 9.8181711574e-03f);
-  p = fmaf(p, x2, -6.6345343288e-02f);
-  p = fmaf(p, x2, 3.9890193482e-01f);
+  float p = 2.7693410957e-08f;
+  p = fmaf(p, x2, -1.8473178272e-06f);
+  p = fmaf(p, x2, 5.2869800351e-05f);
+  p = fmaf(p, x2, -8.6171873090e-04f);
+  p = fmaf(p, x2, 9.0065851481e-03f);
+  p = fmaf(p, x2, -6.5103946404e-02f);
+  p = fmaf(p, x2, 3.9828952833e-01f);
   return x * fmaf(p, xc, 0.5f);
 }
 

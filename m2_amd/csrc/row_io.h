@@ -47,6 +47,13 @@ template <int Q> struct RawRow<float, Q> {
     o[2] = a[I].x + add; o[3] = a[I].y + add; o[4] = a[I].z + add; o[5] = a[I].w + add;
     o[6] = b[I].x + add; o[7] = b[I].y + add; o[8] = b[I].z + add; o[9] = b[I].w + add;
   }
+  // the same without the addend (no add instructions at all)
+  template <int I> __device__ __forceinline__ void expand(int n0, float (&o)[10]) const {
+    o[0] = n0 > 0 ? h[I].x : 0.f;
+    o[1] = n0 > 0 ? h[I].y : 0.f;
+    o[2] = a[I].x; o[3] = a[I].y; o[4] = a[I].z; o[5] = a[I].w;
+    o[6] = b[I].x; o[7] = b[I].y; o[8] = b[I].z; o[9] = b[I].w;
+  }
 };
 template <int Q> struct RawRow<uint16_t, Q> {
   u32x4_t a[Q];
@@ -62,6 +69,14 @@ template <int Q> struct RawRow<uint16_t, Q> {
     o[4] = __uint_as_float(a[I].y << 16) + add; o[5] = __uint_as_float(a[I].y & 0xffff0000u) + add;
     o[6] = __uint_as_float(a[I].z << 16) + add; o[7] = __uint_as_float(a[I].z & 0xffff0000u) + add;
     o[8] = __uint_as_float(a[I].w << 16) + add; o[9] = __uint_as_float(a[I].w & 0xffff0000u) + add;
+  }
+  template <int I> __device__ __forceinline__ void expand(int n0, float (&o)[10]) const {
+    o[0] = n0 > 0 ? __uint_as_float(h[I] << 16) : 0.f;
+    o[1] = n0 > 0 ? __uint_as_float(h[I] & 0xffff0000u) : 0.f;
+    o[2] = __uint_as_float(a[I].x << 16); o[3] = __uint_as_float(a[I].x & 0xffff0000u);
+    o[4] = __uint_as_float(a[I].y << 16); o[5] = __uint_as_float(a[I].y & 0xffff0000u);
+    o[6] = __uint_as_float(a[I].z << 16); o[7] = __uint_as_float(a[I].z & 0xffff0000u);
+    o[8] = __uint_as_float(a[I].w << 16); o[9] = __uint_as_float(a[I].w & 0xffff0000u);
   }
 };
 

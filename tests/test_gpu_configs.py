@@ -157,7 +157,7 @@ def test_config5_wo_wide_tiles(gpu, M):
                                             (32768 - 70, 768, 3072, 3.0)])
 def test_glu_at_benchmark_sizes_and_gelu_tails(gpu, M, d, I, gate_std):
     """The gated GEMM at the M the benchmark runs (configs 3 / 4: M = 32768 at d = 768; config 5: M = 8192 at
-    d = 1536), and with gate pre-activations of standard deviation 3, so that |x| > 4.2 (where the kernel's
+    d = 1536), and with gate pre-activations of standard deviation 3, so that |x| > 3.9 (where the kernel's
     polynomial for x Phi(x) is clamped) and the tails in between are compared with the erf form."""
     from m2_amd import ops
     from oracle import m2_oracle as O
@@ -170,13 +170,13 @@ def test_glu_at_benchmark_sizes_and_gelu_tails(gpu, M, d, I, gate_std):
     h = O.blockdiag_multiply(x.float(), wg.float()).double()
     gate = h[:, :I]
     if gate_std > 1:
-        assert (gate.abs() > 4.2).float().mean() > 0.05          # the clamped range is really exercised
+        assert (gate.abs() > 3.9).float().mean() > 0.05          # the clamped range is really exercised
     ref = torch.nn.functional.gelu(gate) * h[:, I:]
     e, e2 = rel_err(got.float(), ref)
     assert e < TOL_BF16 and e2 < 6e-3, (e, e2)
-    # element-wise: within bf16 rounding (2^-8 relative) plus the polynomial's absolute error times |value|
+    # element-wise: within bf16 rounding (2^-8 relative) plus the polynomial's absolute error (1.8e-4) times |value|
     err = (got.float().cpu().double() - ref).abs()
-    bound = ref.abs() * 2.0 ** -7 + 1e-4 * (h[:, I:].abs() + 1)
+    bound = ref.abs() * 2.0 ** -7 + 2.5e-4 * (h[:, I:].abs() + 1)
     assert bool((err <= bound).all()), float((err - bound).max())
 
 
