@@ -127,25 +127,36 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
         const float wv0 = w[6 * (long)d + 0], wv1 = w[6 * (long)d + 1], wv2 = w[6 * (long)d + 2], bbv = sb[2 * d + c];
         const float w20 = w[3 * (long)d + 0], w21 = w[3 * (long)d + 1], w22 = w[3 * (long)d + 2], bb2 = sb[d + c];
         const float p1 = pbias ? pbias[c] : 0.f, pv = pbias ? pbias[2 * d + c] : 0.f, p2 = pbias ? pbias[d + c] : 0.f;
+        // The bias p of the in-projection is not added to the inputs: a 3-tap convolution of (x + p) is the
+        // convolution of x plus p (w0 + w1 + w2), which goes into the convolution's own bias -- except for the first
+        // two outputs of a row, where one or two taps fall on the zero padding: those are corrected.
+        const float f1 = bb1 + p1 * (w10 + w11 + w12), fv = bbv + pv * (wv0 + wv1 + wv2), f2 = bb2 + p2 * (w20 + w21 + w22);
         __builtin_amdgcn_sched_barrier(0);
-        r1.template expand<0>(n0, p1, in);
+        float cv[8];
+        r1.template expand<0>(n0, in);
         static_for<0, 8>([&](auto jj) {
           constexpr int j = decltype(jj)::value;
-          a[j] = bb1 + w10 * in[j] + w11 * in[j + 1] + w12 * in[j + 2];
+          a[j] = f1 + w10 * in[j] + w11 * in[j + 1] + w12 * in[j + 2];
         });
-        rv.template expand<0>(n0, pv, in);
+        rv.template expand<0>(n0, in);
         static_for<0, 8>([&](auto jj) {
           constexpr int j = decltype(jj)::value;
-          a[j] *= bbv + wv0 * in[j] + wv1 * in[j + 1] + wv2 * in[j + 2];
+          cv[j] = fv + wv0 * in[j] + wv1 * in[j + 1] + wv2 * in[j + 2];
         });
-        r2.template expand<0>(n0, p2, in);
+        r2.template expand<0>(n0, in);
         static_for<0, 8>([&](auto jj) {
           constexpr int j = decltype(jj)::value;
-          gate[j] = bb2 + w20 * in[j] + w21 * in[j + 1] + w22 * in[j + 2];
+          gate[j] = f2 + w20 * in[j] + w21 * in[j + 1] + w22 * in[j + 2];
         });
+        if (n0 == 0) {      // time steps 0 and 1 of the row
+          a[0] -= p1 * (w10 + w11); a[1] -= p1 * w10;
+          cv[0] -= pv * (wv0 + wv1); cv[1] -= pv * wv0;
+          gate[0] -= p2 * (w20 + w21); gate[1] -= p2 * w20;
+        }
+        static_for<0, 8>([&](auto jj) { a[decltype(jj)::value] *= cv[decltype(jj)::value]; });
       } else {
         // plain long convolution: xproj is a single (d, B, L) signal, no short conv, no gates
-        r1.template expand<0>(n0, 0.f, in);
+        r1.template expand<0>(n0, in);
         static_for<0, 8>([&](auto jj) {
           constexpr int j = decltype(jj)::value;
           a[j] = in[j + 2];

@@ -162,6 +162,7 @@ __device__ __forceinline__ void short_conv_slots(const ACT* __restrict__ p, int 
                                                  float add, cf (&out)[32]) {
   typedef typename PairBits<ACT>::type bits;
   constexpr int NB = sizeof(ACT) == 2 ? 32 : 16;      // slots per batch
+  const float fbias = bias + add * (w[0] + w[1] + w[2]);
   static_for<0, 32 / NB>([&](auto hh) {
     constexpr int h0 = decltype(hh)::value * NB;
     bits prev[NB], cur[NB];
@@ -175,11 +176,21 @@ __device__ __forceinline__ void short_conv_slots(const ACT* __restrict__ p, int 
     static_for<0, NB>([&](auto rr) {
       constexpr int r = h0 + decltype(rr)::value;
       const int m = slot_of<P>(t, r / P::R1, r % P::R1);
-      float2 c = expand_pair(cur[r - h0]), q = expand_pair(prev[r - h0]);
-      c.x += add; c.y += add;
-      q.x = m > 0 ? q.x + add : 0.f;
-      q.y = m > 0 ? q.y + add : 0.f;
-      out[r] = {bias + w[0] * q.x + w[1] * q.y + w[2] * c.x, bias + w[0] * q.y + w[1] * c.x + w[2] * c.y};
+      const float2 c = expand_pair(cur[r - h0]);
+      float2 q = expand_pair(prev[r - h0]);
+      if constexpr (r == 0) {      // only slot m = t of register 0 can be slot 0
+        q.x = m > 0 ? q.x : 0.f;
+        q.y = m > 0 ? q.y : 0.f;
+      }
+      // `add` (the in-projection's bias) is folded into the convolution's bias: conv(x + add) = conv(x) + add (w0 + w1 +
+      // w2), except at time steps 0 and 1, where taps fall on the zero padding outside the biased signal
+      out[r] = {fbias + w[0] * q.x + w[1] * q.y + w[2] * c.x, fbias + w[0] * q.y + w[1] * c.x + w[2] * c.y};
+      if constexpr (r == 0) {
+        if (m == 0) {
+          out[r].re -= add * (w[0] + w[1]);
+          out[r].im -= add * w[0];
+        }
+      }
     });
   });
 }
