@@ -176,7 +176,38 @@ def probe_matrix_pipe(iters: int = 4000):
             rows.append({"lds_reads_per_mfma": reads, "valu_per_mfma": valu, "waves_per_simd": wps, "ms": ms,
                          "tflops": tflops, "frac_of_published_peak": tflops / MFMA_BF16_PEAK_TFLOPS})
     return {"probe": "v_mfma_f32_32x32x16_bf16 loop on all compute units", "published_peak_tflops": MFMA_BF16_PEAK_TFLOPS,
-            "rows": rows}
+            "rows": rows, "dft16_pass": probe_dft16_pass()}
+
+
+def probe_dft16_pass(nrows: int = 1024, iters: int = 200):
+    """The radix-16 pass of the L = 8192 half transform on the vector ALU against the same pass as a split-bf16 MFMA
+    product (m2_probe_dft16_pass_fwd): time per pass over `nrows` LDS-resident rows, and how far one MFMA pass is
+    from one vector-ALU pass on the same random rows."""
+    import ctypes
+    from m2_amd._lib import check, lib
+    stream = lambda: torch.cuda.current_stream().cuda_stream
+    x = torch.randn(nrows, 8192, 2, device="cuda:0", generator=torch.Generator(device="cuda:0").manual_seed(1))
+    out = {}
+    one = {}
+    for name, mode in (("valu", 0), ("mfma_split_bf16", 1)):
+        y = x.clone()
+        check(lib.m2_probe_dft16_pass_fwd(mode, 1, nrows, ctypes.c_void_p(y.data_ptr()), stream()))
+        one[name] = y
+        z = (x * 1e-3).clone()
+        check(lib.m2_probe_dft16_pass_fwd(mode, 2, nrows, ctypes.c_void_p(z.data_ptr()), stream()))
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        z = torch.zeros_like(x)                      # zeros stay zeros: no overflow over many unnormalised passes
+        s.record()
+        check(lib.m2_probe_dft16_pass_fwd(mode, iters, nrows, ctypes.c_void_p(z.data_ptr()), stream()))
+        e.record()
+        torch.cuda.synchronize()
+        out[name + "_us_per_pass"] = s.elapsed_time(e) * 1e3 / iters
+    ref = one["valu"].double()
+    out["mfma_vs_valu_max_rel"] = ((one["mfma_split_bf16"].double() - ref).abs().max() / ref.abs().max()).item()
+    out["mfma_vs_valu_l2_rel"] = ((one["mfma_split_bf16"].double() - ref).norm() / ref.norm()).item()
+    out["rows"], out["iters"] = nrows, iters
+    return out
 
 
 def main():

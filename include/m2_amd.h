@@ -228,6 +228,14 @@ int m2_embed_layernorm_fwd(const long long* input_ids, const long long* token_ty
 int m2_probe_mfma_fwd(int lds_reads_per_mfma, int valu_per_mfma, int waves_per_simd, int iters, float* sink,
                       long long* mfma_per_wave, int* waves, void* stream);
 
+/* Measurement aid (no counterpart in the reference): the radix-16 pass (stride 16, with its twiddles) of the L = 8192
+ * half transform used by the long-convolution kernels, repeated `iters` times in place on nrows rows of 8192
+ * complex64 points (rows: device pointer, nrows * 8192 * 2 floats), each row resident in the LDS of one workgroup.
+ * use_mfma == 0: butterflies on the vector ALU (what m2_mixer_core_fwd runs); use_mfma != 0: the same pass as a
+ * product with the real 32 x 32 form of the 16-point DFT matrix on bf16 MFMA, operands split into bf16 high / low
+ * parts (three products).  bench.py --probe times the two against each other and reports their difference. */
+int m2_probe_dft16_pass_fwd(int use_mfma, int iters, int nrows, float* rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -7,7 +7,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "fft_regs.h"
+#include "fft_split.h"
 #include "m2_internal.h"
 
 namespace m2 {
@@ -65,6 +65,110 @@ static int launch_probe(float* sink, int iters, hipStream_t st) {
   return check_launch("probe_mfma");
 }
 
+// ---------------------------------------------------------------------------------------------
+// One pass of the L = 8192 half transform of the long-convolution kernels (the radix-16 pass at stride 16 with its
+// twiddles, fft_split.h: fwd_pass2) done two ways on a row resident in LDS, to be timed against each other:
+//   MFMA = false  the butterflies on the vector ALU, as the mixer core runs them;
+//   MFMA = true   the 16-point DFTs as a product with the 32 x 32 real form of the DFT matrix on
+//                 v_mfma_f32_32x32x16_bf16: Y = F X with X = [Re x; Im x] (32 x 32 groups per product), every
+//                 operand split into a bf16 high and low part and the three leading products summed (hi hi + hi lo
+//                 + lo hi: 16 mantissa bits), the split done on the fly on the vector ALU, twiddles after it.
+// A workgroup owns one row (8192 complex points) and repeats the pass `iters` times in place.
+// ---------------------------------------------------------------------------------------------
+typedef SplitPlan<13, 32, 16> ProbePlan;
+
+template <bool MFMA>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void probe_dft16_kernel(float2* __restrict__ rows, int iters) {
+  typedef ProbePlan P;
+  extern __shared__ float2 plds[];
+  float2* row = plds;
+  float2* tab2 = plds + P::ROW_LDS;
+  const int t = threadIdx.x, wave = t >> 6, lane = t & 63, i32 = lane & 31, half = lane >> 5;
+  float2* g = rows + (long)blockIdx.x * P::L;
+  tab2_init<P>(tab2);
+  for (int i = t; i < P::L; i += 256) row[sphys(i)] = g[i];
+  __syncthreads();
+  if constexpr (!MFMA) {
+    cf x[32];
+    for (int it = 0; it < iters; ++it) {
+      fwd_pass2<P>(x, t, row, tab2);
+      __syncthreads();
+    }
+  } else {
+    // A operands: row r of F (r < 16: Re Y_r = sum_j cos(2 pi j r / 16) Re x_j + sin(..) Im x_j; r >= 16: Im Y_k =
+    // - sin Re x_j + cos Im x_j, k = r - 16), K = 16 kk + 8 half + e: kk = 0 the Re x_j coefficients, kk = 1 Im x_j
+    bf16x8 ahi[2], alo[2];
+    static_for<0, 2>([&](auto kk_) {
+      constexpr int kk = decltype(kk_)::value;
+      float hi[8], lo[8];
+      for (int e = 0; e < 8; ++e) {
+        const int j = 8 * half + e, k = i32 & 15;
+        float sn, cs;
+        sincospif(2.0f * (float)((j * k) & 15) / 16.0f, &sn, &cs);
+        const float f = (i32 < 16) ? (kk == 0 ? cs : sn) : (kk == 0 ? -sn : cs);
+        hi[e] = bf16_to_f32(f32_to_bf16(f));
+        lo[e] = f - hi[e];
+      }
+      u32x4 ph = {pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3]), pack_bf16x2(hi[4], hi[5]), pack_bf16x2(hi[6], hi[7])};
+      u32x4 pl = {pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(lo[4], lo[5]), pack_bf16x2(lo[6], lo[7])};
+      ahi[kk] = __builtin_bit_cast(bf16x8, ph);
+      alo[kk] = __builtin_bit_cast(bf16x8, pl);
+    });
+    for (int it = 0; it < iters; ++it) {
+      // 512 groups of 16 points per pass; a wave takes 128 of them, 32 per product
+      static_for<0, 4>([&](auto ss) {
+        constexpr int set = decltype(ss)::value;
+        const int q = 128 * wave + 32 * set + i32, blk = q >> 4, m = q & 15;
+        float2* pb = row + sphys(blk * 256 + m);
+        float re[8], im[8];
+        static_for<0, 8>([&](auto ee) {
+          constexpr int e = decltype(ee)::value;
+          const float2 v = pb[spoff(16 * e) + (half ? spoff(128) : 0)];
+          re[e] = v.x;
+          im[e] = v.y;
+        });
+        auto split = [&](const float (&x)[8], bf16x8& h8, bf16x8& l8) __attribute__((always_inline)) {
+          uint32_t ph[4], pl[4];
+          static_for<0, 4>([&](auto pp) {
+            constexpr int pi = decltype(pp)::value;
+            ph[pi] = pack_bf16x2(x[2 * pi], x[2 * pi + 1]);
+            const float l0 = x[2 * pi] - __uint_as_float(ph[pi] << 16), l1 = x[2 * pi + 1] - __uint_as_float(ph[pi] & 0xffff0000u);
+            pl[pi] = pack_bf16x2(l0, l1);
+          });
+          u32x4 a = {ph[0], ph[1], ph[2], ph[3]}, b = {pl[0], pl[1], pl[2], pl[3]};
+          h8 = __builtin_bit_cast(bf16x8, a);
+          l8 = __builtin_bit_cast(bf16x8, b);
+        };
+        bf16x8 rh, rl, ih, il;
+        split(re, rh, rl);
+        split(im, ih, il);
+        floatx16 acc;
+        static_for<0, 16>([&](auto vv) { acc[decltype(vv)::value] = 0.f; });
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[0], rh, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[0], rl, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[1], ih, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[1], il, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[0], rh, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[1], ih, acc, 0, 0, 0);
+        // accumulator element 4 a + b: row 8 a + 4 half + b; rows below 16 are Re Y_k, rows 16 + k are Im Y_k
+        static_for<0, 2>([&](auto aa) {
+          constexpr int a = decltype(aa)::value;
+          static_for<0, 4>([&](auto bb) {
+            constexpr int b = decltype(bb)::value;
+            const int k = 8 * a + 4 * half + b;
+            cf y = {acc[4 * a + b], acc[4 * (a + 2) + b]};
+            const float2 w = tab2[k * 16 + m];
+            if (k > 0) y = cmul(y, cf{w.x, w.y});
+            pb[spoff(128 * a + 16 * b) + (half ? spoff(64) : 0)] = make_float2(y.re, y.im);
+          });
+        });
+      });
+      __syncthreads();
+    }
+  }
+  for (int i = t; i < P::L; i += 256) g[i] = row[sphys(i)];
+}
+
 }  // namespace m2
 
 using namespace m2;
@@ -83,4 +187,14 @@ extern "C" int m2_probe_mfma_fwd(int lds_reads_per_mfma, int valu_per_mfma, int 
   M2_PROBE_CASE(0, 0) M2_PROBE_CASE(1, 0) M2_PROBE_CASE(2, 0) M2_PROBE_CASE(1, 4) M2_PROBE_CASE(1, 6) M2_PROBE_CASE(1, 11)
 #undef M2_PROBE_CASE
   return set_error(M2_ERR_UNSUPPORTED, "m2_probe_mfma_fwd: (reads, valu) must be one of (0,0) (1,0) (2,0) (1,4) (1,6) (1,11)");
+}
+
+extern "C" int m2_probe_dft16_pass_fwd(int use_mfma, int iters, int nrows, float* rows, void* stream) {
+  if (!rows || iters <= 0 || nrows <= 0) return set_error(M2_ERR_ARG, "m2_probe_dft16_pass_fwd: null rows or non-positive count");
+  const size_t lds = (size_t)ProbePlan::WG_LDS * sizeof(float2);
+  auto kern = use_mfma ? probe_dft16_kernel<true> : probe_dft16_kernel<false>;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(probe_dft16): %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(kern, dim3(nrows), dim3(256), lds, (hipStream_t)stream, reinterpret_cast<float2*>(rows), iters);
+  return check_launch("probe_dft16");
 }
