@@ -173,14 +173,23 @@ int m2_blockdiag_linear_f32_fwd(const float* x, const float* w, const float* bia
  * chip:  out = blockdiag_multiply(gelu_erf(h[:, :I]) * h[:, I:], w_out) (+ bias) (+ residual),
  * h = blockdiag_multiply(x, w_gated)  (bert/src/bert_layers.py:482-506: gated_layers, act, wo, residual).  Same
  * arithmetic as m2_blockdiag_glu_fwd followed by m2_blockdiag_linear_fwd (bf16 operands, fp32 accumulation, the
- * gated values rounded to bf16 between the two products).  x (M, in_features) bf16; w_gated (nblocks, 2I/nblocks,
- * in/nblocks) bf16; w_out (nblocks, in/nblocks, I/nblocks) bf16; bias (in_features) fp32 or NULL; residual
+ * gated values rounded to bf16 between the two products).
+ * The kernel streams the weights from L2 once per 128-row tile and is bound by that stream, so it reads them from a
+ * packed copy in which every 1 KB the kernel moves at a time is contiguous: m2_mlp_fused_pack writes it, once per
+ * set of weights (w_gated (nblocks, 2I/nblocks, in/nblocks) bf16, gated_layers.weight; w_out (nblocks, in/nblocks,
+ * I/nblocks) bf16, wo.weight; packed: m2_mlp_fused_packed_bytes bytes of device memory, 16-byte aligned; the size is
+ * that of the two weights together).  m2_mlp_fused_fwd: x (M, in_features) bf16; w_packed as written by
+ * m2_mlp_fused_pack for the same in_features / intermediate / nblocks; bias (in_features) fp32 or NULL; residual
  * (M, in_features) bf16 or NULL; out (M, in_features) of out_dtype.  m2_mlp_fused_supported returns 1 for the shapes
- * the kernel is built for (nblocks == 4, in_features == 768, intermediate % 128 == 0); for others the entry point
- * returns M2_ERR_UNSUPPORTED and the caller uses the two separate entry points. */
+ * the kernel is built for (nblocks == 4, in_features == 768, intermediate % 128 == 0); for others
+ * m2_mlp_fused_packed_bytes returns 0, the other two return M2_ERR_UNSUPPORTED and the caller uses the two separate
+ * entry points. */
 int m2_mlp_fused_supported(int in_features, int intermediate, int nblocks);
-int m2_mlp_fused_fwd(const void* x, const void* w_gated, const void* w_out, const float* bias, const void* residual,
-                     void* out, int M, int in_features, int intermediate, int nblocks, int out_dtype, void* stream);
+long m2_mlp_fused_packed_bytes(int in_features, int intermediate, int nblocks);
+int m2_mlp_fused_pack(const void* w_gated, const void* w_out, void* packed, int in_features, int intermediate,
+                      int nblocks, void* stream);
+int m2_mlp_fused_fwd(const void* x, const void* w_packed, const float* bias, const void* residual, void* out, int M,
+                     int in_features, int intermediate, int nblocks, int out_dtype, void* stream);
 
 /* LayerNorm over the last dimension of x (M, d) fp32 (torch.nn.LayerNorm semantics, biased variance,
  * eps inside the root; bert/src/bert_layers.py:478-479,506 and :185-186,247).  Any of the three

@@ -9,24 +9,34 @@
 // and whose paired values come from block r / 2 + 2, so the MLP falls apart into four independent chains
 // x[:, two blocks] -> I/4 gated columns -> 192 output columns, one per r.
 //
-// A workgroup of four waves owns 128 rows and one r.  Everything is computed TRANSPOSED, weights as the MFMA
-// A operand (rows of the product) and the x rows as the B operand (its columns):
+// A workgroup of eight waves (two per SIMD) owns 128 rows and one r; a wave owns 16 rows.  Everything is computed
+// TRANSPOSED, weights as the MFMA A operand (rows of the product) and the x rows as the B operand (its columns),
+// on v_mfma_f32_16x16x32_bf16:
 //
-//   G^T (32 gated columns x 32 x-rows)   = Wg_chunk (32 x 192) X_a^T  and  Wv_chunk X_b^T       24 MFMAs
-//   OUT^T (192 x 32 x-rows)             += Wo_chunk (192 x 32) GLU(G^T)                          12 MFMAs
+//   G^T (32 gated columns x 16 x-rows)   = Wg_chunk (32 x 192) X_a^T  and  Wv_chunk X_b^T       24 MFMAs
+//   OUT^T (192 x 16 x-rows)             += Wo_chunk (192 x 32) GLU(G^T)                          12 MFMAs
 //
-// because then the accumulator of the first product IS the B operand of the second: lane (i, h) of
-// v_mfma_f32_32x32x16_bf16 receives accumulator rows 8 (v / 4) + 4 h + v % 4 of column i, and a B operand wants
-// eight consecutive K values of column i per lane.  Which gated column sits in which accumulator row is free, so
-// operand row rho of a chunk is given gated column gamma(rho) = rho with bits 2 and 3 swapped: then the
-// accumulator elements 8 s .. 8 s + 7 of lane (i, h) are the gated columns 16 s + 8 h .. + 7, exactly the K range
-// of one 16-byte piece of a `wo` row, and the gated values go from the accumulators through gelu(gate) * value
-// and the bf16 conversion straight into the next MFMA: the (M, I) intermediate never leaves the registers.
-// The x rows of a wave (32 rows x two 192-wide blocks = 96 registers) are loaded once, straight from global
-// memory in operand layout, and stay put.  The weights stream through LDS, 36 KB per chunk of 32 gated columns,
-// in three stages, written by direct global -> LDS loads (global_load_lds_dwordx4: no registers, no LDS write
-// instructions) issued two chunks ahead; every operand is one conflict-free 16-byte LDS read (a stage is laid out
-// [K step][lane]).  One barrier per chunk.  One workgroup per compute unit, one wave per SIMD.
+// because then the accumulator of the first product IS the B operand of the second: lane (n, q) of the MFMA
+// receives accumulator rows 4 q .. 4 q + 3 of column n, and a B operand wants the eight K values 8 q .. 8 q + 7
+// of column n.  Which gated column sits in which accumulator row is free, so operand row rho = 16 t + 4 q + j of
+// a chunk (t = row tile) is given gated column gamma(rho) = 8 q + 4 t + j: the eight accumulator elements of a
+// lane (two row tiles x four) are then the gated columns 8 q .. 8 q + 7, exactly the K range of one 16-byte piece
+// of a `wo` row, and the gated values go from the accumulators through gelu(gate) * value and the bf16
+// conversion straight into the next MFMA: the (M, I) intermediate never leaves the registers.
+// The x rows of a wave (16 rows x two 192-wide blocks = 48 registers) are loaded once per row tile, straight from
+// global memory in operand layout, and stay put.  The weights stream through LDS, 36 KB per chunk of 32 gated
+// columns, in four stages, written by direct global -> LDS loads (global_load_lds_dwordx4: no registers, no LDS
+// write instructions) issued three chunks ahead; every operand is one conflict-free 16-byte LDS read (a stage is
+// laid out [operand block][lane]).  One barrier per chunk; the operand reads run ahead of the MFMAs through a ring
+// of registers that does not drain at the barrier (the next chunk is complete one barrier early).
+//
+// Every compute unit streams ALL weights of its r once per 128-row tile, from L2: 36 KB per 0.5 us of MFMA work, and
+// that stream, not the matrix pipe, is what bounds the kernel.  Measured on MI355X with all 256 compute units
+// streaming (direct-to-LDS loads, L2 hits): 62 GB/s per compute unit when a load instruction covers 1 KB of
+// contiguous memory, 38 GB/s when it gathers sixteen 64-byte row pieces (the operand layout taken straight from the
+// row-major weights).  So the weights are re-packed once (m2_mlp_fused_pack) into the exact image of the LDS
+// stages -- per (r, chunk) 36 operand blocks of 1 KB, lane-major -- and every load instruction copies one contiguous
+// block.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -37,7 +47,7 @@
 
 namespace m2 {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -58,18 +68,20 @@ __device__ __forceinline__ float gelu_erf_poly(float x) {
 }
 
 constexpr int kFP = 192;                    // block width of x and of the output (d / 4)
-constexpr int kFKS = kFP / 16;              // K steps of the first products: 12
-constexpr int kFRows = 128;                 // rows per workgroup
+constexpr int kFKS = kFP / 32;              // K steps of the first products (K = 32 per MFMA): 6
+constexpr int kFRows = 128;                 // rows per workgroup: 8 waves x 16
 constexpr int kFChunk = 32;                 // gated columns per chunk
-constexpr int kFBlk = 1024;                 // one operand block: 64 lanes x 16 bytes
-constexpr int kFGV = 2 * kFKS * kFBlk;      // Wg + Wv blocks of a chunk: 24 KB
-constexpr int kFWO = 12 * kFBlk;            // Wo blocks of a chunk (6 tiles x 2 K steps): 12 KB
-constexpr int kFStages = 3;
-constexpr int kFLds = kFStages * (kFGV + kFWO);      // 108 KB
+constexpr int kFBlk = 1024;                 // one operand block: 64 lanes x 16 bytes = 16 rows x 32 K
+constexpr int kFGV = 2 * 2 * kFKS * kFBlk;  // Wg + Wv of a chunk: (gate | value) x 2 row tiles x 6 K steps = 24 KB
+constexpr int kFWO = 12 * kFBlk;            // Wo of a chunk: 12 output tiles of 16 columns = 12 KB
+constexpr int kFStages = 4;
+constexpr int kFLds = kFStages * (kFGV + kFWO);      // 144 KB
+constexpr int kFChunkBytes = kFGV + kFWO;   // a chunk in the packed weights: the image of its two stages
+constexpr int kFBatch = 5;                  // direct loads a wave issues per chunk: 3 (Wg / Wv) + 2 (Wo; 1 for waves 4 .. 7)
 
 // s_waitcnt immediates (vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8): wait for the vector-memory
 // counter only
-constexpr int kWaitVm0 = 0x0F70, kWaitVm9 = 0x0F79;
+constexpr int kWaitVm0 = 0x0F70, kWaitVmBatch = 0x0F70 | kFBatch, kWaitVmBatch1 = 0x0F70 | (kFBatch - 1);
 
 // One direct global -> LDS load: every lane fetches 16 bytes from base + voff, lane l's piece lands at LDS byte
 // address lds + 16 l.  Inline assembly on purpose: the compiler then neither tracks the LDS write (it would put a
@@ -79,226 +91,220 @@ __device__ __forceinline__ void load_to_lds(unsigned lds, unsigned voff, const v
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(base) : "memory");
 }
 
+// Re-packs gated_layers.weight (4, I / 2, 192) and wo.weight (4, 192, I / 4) into the image of the LDS stages: for
+// r = 0 .. 3 and chunk c (32 gated columns) 24 Wg / Wv blocks and 12 Wo blocks of 64 lanes x 16 bytes.  One thread
+// per 16-byte piece.  Lane (i, q) of Wg / Wv block ((value, t), s) holds row gamma(16 t + i) = 8 (i / 4) + 4 t + i % 4
+// of the chunk, K = 32 s + 8 q .. + 7; of Wo block tau row 16 tau + i, K = 8 q .. + 7 of the chunk.
+__global__ __launch_bounds__(256) void mlp_fused_pack_kernel(const uint16_t* __restrict__ wg, const uint16_t* __restrict__ wo,
+                                                             u32x4* __restrict__ packed, int I) {
+  const int IS = I >> 2, q = I >> 1, nchunks = IS / kFChunk;
+  const long piece = (long)blockIdx.x * 256 + threadIdx.x;
+  const long npieces = 4l * nchunks * (kFChunkBytes / 16);
+  if (piece >= npieces) return;
+  const int lane = piece & 63, i16 = lane & 15, q4 = lane >> 4;
+  const int blk = (piece >> 6) % 36;
+  const int c = (piece / (64 * 36)) % nchunks;
+  const int r = piece / (64l * 36 * nchunks);
+  const uint16_t* src;
+  if (blk < 24) {
+    const int s = blk % kFKS, t = (blk / kFKS) & 1, val = blk / (2 * kFKS);
+    const int gamma = 8 * (i16 >> 2) + 4 * t + (i16 & 3);
+    src = wg + (((long)((r >> 1) + 2 * val) * q + (long)(r & 1) * IS + c * kFChunk + gamma) * kFP + 32 * s + 8 * q4);
+  } else {
+    src = wo + (((long)r * kFP + 16 * (blk - 24) + i16) * IS + c * kFChunk + 8 * q4);
+  }
+  packed[piece] = *reinterpret_cast<const u32x4*>(src);
+}
+
 template <typename OUT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlp_fused_kernel(
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mlp_fused_kernel(
     const uint16_t* __restrict__ x,       // (M, 768) bf16
-    const uint16_t* __restrict__ wg,      // (4, I / 2, 192) bf16   gated_layers.weight
-    const uint16_t* __restrict__ wo,      // (4, 192, I / 4) bf16   wo.weight
+    const unsigned char* __restrict__ wpk,      // both weights as packed by mlp_fused_pack_kernel
     const float* __restrict__ bias,       // (768) or null
     const uint16_t* __restrict__ resid,   // (M, 768) bf16 or null
     OUT* __restrict__ out,                // (M, 768)
-    int M, int I) {
+    int M, int I, int ntiles) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, i16 = lane & 15, q4 = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): XCD e works on output block r = e % 4 only,
-  // so its L2 holds one quarter of the weights.
+  // so its L2 holds one quarter of the weights, and on the row tiles of parity e / 4.  A workgroup is persistent:
+  // it walks over its row tiles while the weight stream through LDS just keeps cycling.
   const int xcd = blockIdx.x & 7;
   const int r = xcd & 3;
-  const int tile = (blockIdx.x >> 3) * 2 + (xcd >> 2);
-  const int m0 = tile * kFRows;
-  if (m0 >= M) return;
+  const int tile_step = 2 * (int)(gridDim.x >> 3);
+  int tile = 2 * (int)(blockIdx.x >> 3) + (xcd >> 2);
+  if (tile >= ntiles) return;
   const int IS = I >> 2;                  // gated columns of this r
-  const int q = I >> 1;                   // rows of a gated_layers block
   const int nchunks = IS / kFChunk;
   const int gb = r >> 1;                  // gate block; the value block is gb + 2
   const int d = 4 * kFP;
 
-  // ---- the wave's x rows as stationary B operands: lane (i, h) holds x[row i][16 s + 8 h .. + 8) of both blocks
+  // ---- the wave's x rows as stationary B operands: lane (n, q) holds x[row n][32 s + 8 q .. + 8) of both blocks
   bf16x8 xa[kFKS], xb[kFKS];
-  {
-    int row = m0 + 32 * wave + i32;
+  auto load_x = [&](int t) __attribute__((always_inline)) {
+    int row = t * kFRows + 16 * wave + i16;
     row = row < M ? row : M - 1;
-    const uint16_t* pa = x + (long)row * d + gb * kFP + 8 * half;
+    const uint16_t* pa = x + (long)row * d + gb * kFP + 8 * q4;
     const uint16_t* pb = pa + 2 * kFP;
     static_for<0, kFKS>([&](auto ss) {
       constexpr int s = decltype(ss)::value;
-      xa[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pa + 16 * s));
-      xb[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pb + 16 * s));
+      xa[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pa + 32 * s));
+      xb[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pb + 32 * s));
     });
-  }
+  };
+  load_x(tile);
 
-  // ---- staging.  A chunk is 36 operand blocks of 1 KB: Wg K steps 0 .. 11, Wv K steps 0 .. 11, Wo (tile t, K step
-  // s2) 0 .. 11; wave w loads the blocks b = w + 4 j.  Lane (i, h) of a block fetches what lane (i, h) of the MFMA
-  // needs: Wg / Wv row gamma(i) of the chunk, K = 16 s + 8 h .. + 7; Wo row 32 t + i, K = 16 s2 + 8 h .. + 7.
+  // ---- staging.  The packed weights hold, per (r, chunk), 36 operand blocks of 1 KB, lane-major: Wg / Wv block
+  // ((value, row tile t), K step s) = index (2 value + t) 6 + s, then Wo blocks tau = 0 .. 11 (output columns
+  // [16 tau, + 16)); lane (i, q) of a block holds what lane (i, q) of the MFMA needs.  Wave w copies the Wg / Wv blocks
+  // w, w + 8, w + 16, the Wo block w and, for w < 4, the Wo block w + 8.
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
-  const int gamma = (i32 & 0x13) | ((i32 & 4) << 1) | ((i32 & 8) >> 1);
-  unsigned voff_gv[6], voff_o[3];
-  static_for<0, 6>([&](auto jj) {
+  const unsigned voff = 16 * lane;
+  const unsigned char* wr = wpk + (long)r * nchunks * kFChunkBytes;
+  // Iterations are counted through all tiles of the workgroup (n = 0, 1, ...); iteration n reads Wg / Wv from stage
+  // n % 4 and Wo from stage (n - 1) % 4.
+  auto stage_gv = [&](int n) { return (n & (kFStages - 1)) * kFGV; };
+  auto stage_wo = [&](int n) { return kFStages * kFGV + ((n - 1) & (kFStages - 1)) * kFWO; };
+  // Load j of the batch that feeds iteration n, which is iteration `it` (0 .. nchunks) of its tile: Wg / Wv of chunk
+  // `it` (iteration nchunks only repeats the last chunk) or Wo of chunk it - 1 (iteration 0 multiplies zeros by
+  // whatever finite numbers it finds: chunk 0).
+  auto dma_one = [&](int n, int it, auto jj) __attribute__((always_inline)) {
     constexpr int j = decltype(jj)::value;
-    const int b = wave + 4 * j, s = b % kFKS, val = b / kFKS;
-    voff_gv[j] = (unsigned)((((long)(gb + 2 * val) * q + (long)(r & 1) * IS + gamma) * kFP + 16 * s + 8 * half) * 2);
-  });
-  static_for<0, 3>([&](auto jj) {
-    constexpr int j = decltype(jj)::value;
-    const int b = wave + 4 * j, t = b >> 1, s2 = b & 1;
-    voff_o[j] = (unsigned)((((long)r * kFP + 32 * t + i32) * IS + 16 * s2 + 8 * half) * 2);
-  });
-  auto stage_gv = [&](int c) { return lds0 + (c % kFStages) * kFGV; };
-  auto stage_wo = [&](int c) { return lds0 + kFStages * kFGV + (c % kFStages) * kFWO; };
-  // Wg / Wv of chunk c -> its stage (indices past the end are clamped: nobody reads what that fetches)
-  auto dma_gv = [&](int c) __attribute__((always_inline)) {
-    const unsigned st = __builtin_amdgcn_readfirstlane(stage_gv(c) + wave * kFBlk);
-    const int cc = c < nchunks ? c : nchunks - 1;
-    const uint16_t* base = wg + (long)cc * kFChunk * kFP;
-    static_for<0, 6>([&](auto jj) { load_to_lds(st + 4 * kFBlk * decltype(jj)::value, voff_gv[decltype(jj)::value], base); });
-  };
-  auto dma_wo = [&](int c) __attribute__((always_inline)) {
-    const unsigned st = __builtin_amdgcn_readfirstlane(stage_wo(c) + wave * kFBlk);
-    const int cc = c < nchunks ? c : nchunks - 1;
-    const uint16_t* base = wo + cc * kFChunk;
-    static_for<0, 3>([&](auto jj) { load_to_lds(st + 4 * kFBlk * decltype(jj)::value, voff_o[decltype(jj)::value], base); });
+    if constexpr (j < 3) {
+      const int cc = it < nchunks ? it : nchunks - 1;
+      load_to_lds(lds0 + stage_gv(n) + (wave + 8 * j) * kFBlk, voff, wr + (long)cc * kFChunkBytes + (wave + 8 * j) * kFBlk);
+    } else {
+      const int cc = it > 0 ? it - 1 : 0;
+      const int tau = wave + 8 * (j - 3);
+      if (j == 3 || wave < 4)
+        load_to_lds(lds0 + stage_wo(n) + tau * kFBlk, voff, wr + (long)cc * kFChunkBytes + kFGV + tau * kFBlk);
+    }
   };
 
-  floatx16 acc_out[6];
-  static_for<0, 6>([&](auto tt) {
-    static_for<0, 16>([&](auto vv) { acc_out[decltype(tt)::value][decltype(vv)::value] = 0.f; });
-  });
+  floatx4 acc_out[12];
+  floatx4 g[2], v[2];
+  float gp[8], vp[8];      // the previous chunk's gate / value accumulators, in gated-column order 4 t + j
 
-  // The instruction stream of an iteration is laid out by hand and pinned with scheduling barriers (one wave per
-  // SIMD: nothing else hides a latency).  LDS operand reads run kPF MFMAs ahead through a ring of registers; the
-  // MFMAs of the first products of chunk i carry the vector-ALU work of gelu(gate) * value of chunk i - 1.
-  constexpr int kPF = 6;
-  constexpr int kNP = 2 * kFKS;       // MFMAs of the first products per chunk: 24
-
-  auto gelu_pack = [&](const float (&gl)[16], bf16x8 (&gt)[2]) __attribute__((always_inline)) {
-    static_for<0, 2>([&](auto ss) {
-      constexpr int s = decltype(ss)::value;
-      u32x4 pk;
-      pk.x = pack_bf16x2(gl[8 * s + 0], gl[8 * s + 1]);
-      pk.y = pack_bf16x2(gl[8 * s + 2], gl[8 * s + 3]);
-      pk.z = pack_bf16x2(gl[8 * s + 4], gl[8 * s + 5]);
-      pk.w = pack_bf16x2(gl[8 * s + 6], gl[8 * s + 7]);
-      gt[s] = __builtin_bit_cast(bf16x8, pk);
-    });
+  // ---- the instruction stream of an iteration: 36 MFMAs, laid out by hand and pinned with scheduling barriers.
+  // MFMA k < 24: first products of chunk i, K step k / 4, (gate t = 0, value t = 0, gate t = 1, value t = 1) = k % 4;
+  // MFMA 24 + tau: OUT^T tile tau += Wo block tau of chunk i - 1 times gelu * value of chunk i - 1.
+  // The operand of MFMA k + kPF is read right after MFMA k is issued; past the end of the iteration those are the
+  // first operands of the next one (its chunk has been complete in LDS since the last barrier).
+  constexpr int kNM = 36;
+  constexpr int kPF = 12;      // divides kNM, so that operand k of every iteration sits in ring slot k % kPF
+  static_assert(kNM % kPF == 0, "the ring must close over an iteration");
+  const unsigned char* lane_base = smem + 16 * lane;
+  auto operand_addr = [&](int n, auto kk) __attribute__((always_inline)) -> const unsigned char* {
+    constexpr int k = decltype(kk)::value;
+    if constexpr (k < 24) {
+      constexpr int s = k / 4, sel = k % 4, t = sel >> 1, val = sel & 1;
+      return lane_base + stage_gv(n) + ((2 * val + t) * kFKS + s) * kFBlk;
+    } else {
+      return lane_base + stage_wo(n) + (k - 24) * kFBlk;
+    }
   };
+  u32x4 ring[kPF];
+  bf16x8 gt;
 
-  // first products of chunk i into (g, v); with GLU: gelu * value of chunk i - 1, whose accumulators were copied
-  // to (gp, vp) -> gt
-  auto first_phase = [&](int i, floatx16& g, floatx16& v, const float (&gp)[16], const float (&vp)[16], bf16x8 (&gt)[2],
-                         auto with_glu) __attribute__((always_inline)) {
-    constexpr bool GLU = decltype(with_glu)::value;
-    const unsigned char* ag = smem + (i % kFStages) * kFGV + 16 * lane;
-    // MFMA k: K step k / 2 of the gate (k even) or value (k odd) product
-    auto addr = [&](auto kk) __attribute__((always_inline)) {
-      constexpr int k = decltype(kk)::value;
-      return ag + ((k & 1) * kFKS + (k >> 1)) * kFBlk;
-    };
-    u32x4 ring[kPF];
-    static_for<0, kPF>([&](auto kk) { ring[decltype(kk)::value] = *reinterpret_cast<const u32x4*>(addr(kk)); });
-    float gl[16];
-    __builtin_amdgcn_sched_barrier(0);
-    static_for<0, kNP>([&](auto kk) {
-      constexpr int k = decltype(kk)::value;
-      const bf16x8 a = __builtin_bit_cast(bf16x8, ring[k % kPF]);
-      if constexpr (k == 0) {
-        floatx16 z;
-        static_for<0, 16>([&](auto vv) { z[decltype(vv)::value] = 0.f; });
-        g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xa[0], z, 0, 0, 0);
-      } else if constexpr (k == 1) {
-        floatx16 z;
-        static_for<0, 16>([&](auto vv) { z[decltype(vv)::value] = 0.f; });
-        v = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xb[0], z, 0, 0, 0);
-      } else if constexpr ((k & 1) == 0) {
-        g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xa[k >> 1], g, 0, 0, 0);
-      } else {
-        v = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, xb[k >> 1], v, 0, 0, 0);
-      }
-      if constexpr (k + kPF < kNP) ring[k % kPF] = *reinterpret_cast<const u32x4*>(addr(ic<k + kPF>{}));
-      if constexpr (GLU && k < 16) gl[k] = gelu_erf_poly(gp[k]) * vp[k];
-      __builtin_amdgcn_sched_barrier(0);
-    });
-    if constexpr (GLU) gelu_pack(gl, gt);
-  };
-  // second product: OUT^T += Wo_chunk (chunk c) * G^T; MFMA k = K step k / 6 of output tile k % 6, so that
-  // consecutive MFMAs write different accumulators.  Along with it the accumulators (g, v) of the first products
-  // just finished are copied out to (gp, vp) for the next iteration's gelu * value.
-  auto second_phase = [&](int c, const bf16x8 (&gt)[2], const floatx16& g, const floatx16& v, float (&gp)[16],
-                          float (&vp)[16], auto with_copy) __attribute__((always_inline)) {
-    constexpr bool COPY = decltype(with_copy)::value;
-    const unsigned char* ao = smem + kFStages * kFGV + (c % kFStages) * kFWO + 16 * lane;
-    auto addr = [&](auto kk) __attribute__((always_inline)) {
-      constexpr int k = decltype(kk)::value;
-      return ao + ((k % 6) * 2 + k / 6) * kFBlk;
-    };
-    u32x4 ring[kPF];
-    static_for<0, kPF>([&](auto kk) { ring[decltype(kk)::value] = *reinterpret_cast<const u32x4*>(addr(kk)); });
-    __builtin_amdgcn_sched_barrier(0);
-    static_for<0, 12>([&](auto kk) {
-      constexpr int k = decltype(kk)::value;
-      acc_out[k % 6] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ring[k % kPF]), gt[k / 6],
-                                                               acc_out[k % 6], 0, 0, 0);
-      if constexpr (k + kPF < 12) ring[k % kPF] = *reinterpret_cast<const u32x4*>(addr(ic<k + kPF>{}));
-      if constexpr (COPY && k >= 4) {
-        static_for<4 * (k - 4), 4 * (k - 3)>([&](auto ee) {
-          constexpr int e = decltype(ee)::value;
-          if constexpr (e < 16) gp[e] = g[e];
-          else vp[e - 16] = v[e - 16];
-        });
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    });
-  };
-
-  // ---- pipeline.  Batch i of loads, issued at the top of iteration i: Wg / Wv of chunk i + 2 into the stage last
-  // read as chunk i - 1 (before the barrier of iteration i), Wo of chunk i + 1 into the stage last read as chunk
-  // i - 2 (Wo of chunk c is consumed one iteration later than its Wg / Wv, in iteration c + 1).  Before it reaches
-  // the barrier of iteration i + 1 a wave waits until at most its newest batch is in flight, so batch i - 1 (Wg / Wv
-  // of chunk i + 1, Wo of chunk i) is in LDS for everybody after that barrier.
-  dma_gv(0);
-  dma_gv(1);
-  dma_wo(0);
-  floatx16 g, v;
-  float gp[16], vp[16];
-  bf16x8 gt[2];
-  __builtin_amdgcn_s_waitcnt(kWaitVm0);
-
-  // iteration 0: only the first products of chunk 0
-  __syncthreads();
-  dma_gv(2);
-  dma_wo(1);
-  first_phase(0, g, v, gp, vp, gt, std::false_type{});
-  static_for<0, 16>([&](auto ee) { gp[decltype(ee)::value] = g[decltype(ee)::value]; vp[decltype(ee)::value] = v[decltype(ee)::value]; });
-  __builtin_amdgcn_s_waitcnt(kWaitVm9);
-  for (int i = 1; i < nchunks; ++i) {
-    __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();
-    __builtin_amdgcn_sched_barrier(0);
-    dma_gv(i + 2);
-    dma_wo(i + 1);
-    __builtin_amdgcn_sched_barrier(0);
-    first_phase(i, g, v, gp, vp, gt, std::true_type{});
-    __builtin_amdgcn_sched_barrier(0);
-    second_phase(i - 1, gt, g, v, gp, vp, std::true_type{});
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(kWaitVm9);
+  // prologue: the batches of iterations 0 .. 2; then the ring for iteration 0
+  int it3 = 0;             // which iteration of its tile iteration n + 3 is
+  for (int n = 0; n < 3; ++n) {
+    static_for<0, kFBatch>([&](auto jj) { dma_one(n, it3, jj); });
+    it3 = it3 == nchunks ? 0 : it3 + 1;
   }
-  // last iteration: gelu * value and the second product of the last chunk.  No load may still be in flight when
-  // the workgroup ends (its LDS goes to the next one).
   __builtin_amdgcn_s_waitcnt(kWaitVm0);
   __syncthreads();
+  static_for<0, kPF>([&](auto kk) { ring[decltype(kk)::value] = *reinterpret_cast<const u32x4*>(operand_addr(0, kk)); });
   {
-    float gl[16];
-    static_for<0, 16>([&](auto kk) { gl[decltype(kk)::value] = gelu_erf_poly(gp[decltype(kk)::value]) * vp[decltype(kk)::value]; });
-    gelu_pack(gl, gt);
+    u32x4 z = {0u, 0u, 0u, 0u};
+    gt = __builtin_bit_cast(bf16x8, z);
   }
-  second_phase(nchunks - 1, gt, g, v, gp, vp, std::false_type{});
 
-  // ---- epilogue: accumulator element v = 4 a + b of tile t is output column 32 t + 8 a + 4 h + b of x-row i
-  const int row = m0 + 32 * wave + i32;
-  if (row < M) {
-    const long o0 = (long)row * d + r * kFP + 4 * half;
-    static_for<0, 6>([&](auto tt) {
-      constexpr int t = decltype(tt)::value;
-      static_for<0, 4>([&](auto aa) {
-        constexpr int a = decltype(aa)::value;
-        const int col = 32 * t + 8 * a;
-        float4 val = make_float4(acc_out[t][4 * a], acc_out[t][4 * a + 1], acc_out[t][4 * a + 2], acc_out[t][4 * a + 3]);
+  int n = 0;
+  for (;;) {
+    static_for<0, 12>([&](auto tt) {
+      static_for<0, 4>([&](auto vv) { acc_out[decltype(tt)::value][decltype(vv)::value] = 0.f; });
+    });
+    static_for<0, 8>([&](auto ee) { gp[decltype(ee)::value] = 0.f; vp[decltype(ee)::value] = 0.f; });
+    // The x loads complete here, once per tile: consumed before the loop, the compiler has no reason to keep a
+    // "load may be pending" mark on the x registers around the loop's back edge (that would put a full
+    // vector-memory wait, which also waits for the direct-to-LDS loads just issued, into every iteration).
+#pragma unroll
+    for (int s = 0; s < kFKS; ++s) asm volatile("" : "+v"(xa[s]), "+v"(xb[s]));
+
+    // Iteration i = 0 .. nchunks of the tile.  Iteration 0 has no previous chunk (gelu * value of zeros is zero, the
+    // second product adds nothing); iteration nchunks repeats the first products of the last chunk for nothing: both
+    // keep the loop body free of branches at 1 / nchunks more MFMAs.
+    for (int i = 0; i <= nchunks; ++i, ++n) {
+      float gl[8];
+      static_for<0, kNM>([&](auto kk) {
+        constexpr int k = decltype(kk)::value;
+        const bf16x8 a = __builtin_bit_cast(bf16x8, ring[k % kPF]);
+        if constexpr (k < 24) {
+          constexpr int s = k / 4, sel = k % 4, t = sel >> 1, val = sel & 1;
+          floatx4& acc = val ? v[t] : g[t];
+          if constexpr (s == 0) {
+            const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, val ? xb[0] : xa[0], z, 0, 0, 0);
+          } else {
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, val ? xb[s] : xa[s], acc, 0, 0, 0);
+          }
+        } else {
+          acc_out[k - 24] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, gt, acc_out[k - 24], 0, 0, 0);
+        }
+        // next operand: this iteration's while k + kPF < 36, else the next iteration's
+        if constexpr (k + kPF < kNM) ring[k % kPF] = *reinterpret_cast<const u32x4*>(operand_addr(n, ic<k + kPF>{}));
+        else ring[k % kPF] = *reinterpret_cast<const u32x4*>(operand_addr(n + 1, ic<k + kPF - kNM>{}));
+        // The batch of direct loads for iteration n + 3, one load every seventh MFMA: Wg / Wv into the stage last
+        // read in iteration n - 1, Wo into the one last read in iteration n - 1 as well, both before the barrier that
+        // started this iteration.  (Issued together at the top, the loads of the workgroup fill the memory
+        // pipeline's queue and every wave stalls behind its own loads: 21 us of 210 at M = 32768.)
+        if constexpr (k % 7 == 1 && k / 7 < kFBatch) dma_one(n + 3, it3, ic<k / 7>{});
+        // vector-ALU work riding along: gelu * value of the previous chunk (one element per 3 MFMAs of the first
+        // products), then its packing; during the second product the accumulators just finished are copied out
+        if constexpr (k < 24 && k % 3 == 0) gl[k / 3] = gelu_erf_poly(gp[k / 3]) * vp[k / 3];
+        if constexpr (k == 23) {
+          u32x4 pk;
+          pk.x = pack_bf16x2(gl[0], gl[1]);
+          pk.y = pack_bf16x2(gl[2], gl[3]);
+          pk.z = pack_bf16x2(gl[4], gl[5]);
+          pk.w = pack_bf16x2(gl[6], gl[7]);
+          gt = __builtin_bit_cast(bf16x8, pk);
+        }
+        if constexpr (k >= 28) {
+          constexpr int e = k - 28;      // 0 .. 7: element 4 t + j
+          gp[e] = g[e >> 2][e & 3];
+          vp[e] = v[e >> 2][e & 3];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      it3 = it3 == nchunks ? 0 : it3 + 1;
+      // before the barrier: everything but this wave's newest batch has landed, so after the barrier the chunks of
+      // iterations n + 1 and n + 2 are complete for everybody
+      if (wave < 4) __builtin_amdgcn_s_waitcnt(kWaitVmBatch);
+      else __builtin_amdgcn_s_waitcnt(kWaitVmBatch1);
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- end of the tile: the next tile's x rows are requested first, then this tile's results leave.
+    // Accumulator element j of tile tau is output column 16 tau + 4 q + j of x-row n.
+    const int row = tile * kFRows + 16 * wave + i16;
+    tile += tile_step;
+    const bool more = tile < ntiles;
+    if (more) load_x(tile);
+    if (row < M) {
+      const long o0 = (long)row * d + r * kFP + 4 * q4;
+      static_for<0, 12>([&](auto tt) {
+        constexpr int t = decltype(tt)::value;
+        float4 val = make_float4(acc_out[t][0], acc_out[t][1], acc_out[t][2], acc_out[t][3]);
         if (bias) {
-          const float4 bq = *reinterpret_cast<const float4*>(bias + r * kFP + 4 * half + col);
+          const float4 bq = *reinterpret_cast<const float4*>(bias + r * kFP + 4 * q4 + 16 * t);
           val.x += bq.x; val.y += bq.y; val.z += bq.z; val.w += bq.w;
         }
         if (resid) {
-          const uint2 rr = *reinterpret_cast<const uint2*>(resid + o0 + col);
+          const uint2 rr = *reinterpret_cast<const uint2*>(resid + o0 + 16 * t);
           val.x += __uint_as_float(rr.x << 16); val.y += __uint_as_float(rr.x & 0xffff0000u);
           val.z += __uint_as_float(rr.y << 16); val.w += __uint_as_float(rr.y & 0xffff0000u);
         }
@@ -306,13 +312,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           uint2 pk;
           pk.x = pack_bf16x2(val.x, val.y);
           pk.y = pack_bf16x2(val.z, val.w);
-          *reinterpret_cast<uint2*>(out + o0 + col) = pk;
+          *reinterpret_cast<uint2*>(out + o0 + 16 * t) = pk;
         } else {
-          *reinterpret_cast<float4*>(out + o0 + col) = val;
+          *reinterpret_cast<float4*>(out + o0 + 16 * t) = val;
         }
       });
-    });
+    }
+    if (!more) break;
   }
+  // no load may still be in flight when the workgroup ends (its LDS goes to the next one)
+  __builtin_amdgcn_s_waitcnt(kWaitVm0);
 }
 
 }  // namespace m2
@@ -323,10 +332,27 @@ extern "C" int m2_mlp_fused_supported(int in_features, int intermediate, int nbl
   return nblocks == 4 && in_features == 4 * kFP && intermediate > 0 && intermediate % (4 * kFChunk) == 0;
 }
 
-extern "C" int m2_mlp_fused_fwd(const void* x, const void* w_gated, const void* w_out, const float* bias,
-                                const void* residual, void* out, int M, int in_features, int intermediate, int nblocks,
-                                int out_dtype, void* stream) {
-  if (!x || !w_gated || !w_out || !out) return set_error(M2_ERR_ARG, "m2_mlp_fused_fwd: null pointer");
+extern "C" long m2_mlp_fused_packed_bytes(int in_features, int intermediate, int nblocks) {
+  if (!m2_mlp_fused_supported(in_features, intermediate, nblocks)) return 0;
+  return 4l * (intermediate / 4 / kFChunk) * kFChunkBytes;      // = 2 bytes x (elements of w_gated + elements of w_out)
+}
+
+extern "C" int m2_mlp_fused_pack(const void* w_gated, const void* w_out, void* packed, int in_features, int intermediate,
+                                 int nblocks, void* stream) {
+  if (!w_gated || !w_out || !packed) return set_error(M2_ERR_ARG, "m2_mlp_fused_pack: null pointer");
+  if (!m2_mlp_fused_supported(in_features, intermediate, nblocks))
+    return set_error(M2_ERR_UNSUPPORTED,
+                     "m2_mlp_fused_pack: built for nblocks=4, in_features=768 and intermediate a multiple of 128 "
+                     "(got nblocks=%d in=%d intermediate=%d)", nblocks, in_features, intermediate);
+  const long npieces = m2_mlp_fused_packed_bytes(in_features, intermediate, nblocks) / 16;
+  hipLaunchKernelGGL(mlp_fused_pack_kernel, dim3((unsigned)((npieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t*)w_gated, (const uint16_t*)w_out, (u32x4*)packed, intermediate);
+  return check_launch("mlp_fused_pack");
+}
+
+extern "C" int m2_mlp_fused_fwd(const void* x, const void* w_packed, const float* bias, const void* residual, void* out,
+                                int M, int in_features, int intermediate, int nblocks, int out_dtype, void* stream) {
+  if (!x || !w_packed || !out) return set_error(M2_ERR_ARG, "m2_mlp_fused_fwd: null pointer");
   if (M <= 0) return set_error(M2_ERR_ARG, "m2_mlp_fused_fwd: M=%d must be positive", M);
   if (out_dtype != M2_DTYPE_F32 && out_dtype != M2_DTYPE_BF16)
     return set_error(M2_ERR_ARG, "m2_mlp_fused_fwd: out_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", out_dtype);
@@ -336,20 +362,23 @@ extern "C" int m2_mlp_fused_fwd(const void* x, const void* w_gated, const void* 
                      "(got nblocks=%d in=%d intermediate=%d); use m2_blockdiag_glu_fwd + m2_blockdiag_linear_fwd",
                      nblocks, in_features, intermediate);
   const int ntiles = (M + kFRows - 1) / kFRows;
-  const dim3 grid(8 * ((ntiles + 1) / 2));
+  // one persistent workgroup per compute unit (144 KB of LDS each), 8 per step so that every XCD gets its share
+  int per_xcd = num_cus() / 8;
+  if (per_xcd > (ntiles + 1) / 2) per_xcd = (ntiles + 1) / 2;
+  const dim3 grid(8 * per_xcd);
   hipStream_t st = (hipStream_t)stream;
   if (out_dtype == M2_DTYPE_F32) {
     auto kern = mlp_fused_kernel<float>;
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kFLds);
     if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(mlp_fused): %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, grid, dim3(256), kFLds, st, (const uint16_t*)x, (const uint16_t*)w_gated, (const uint16_t*)w_out,
-                       bias, (const uint16_t*)residual, (float*)out, M, intermediate);
+    hipLaunchKernelGGL(kern, grid, dim3(512), kFLds, st, (const uint16_t*)x, (const unsigned char*)w_packed,
+                       bias, (const uint16_t*)residual, (float*)out, M, intermediate, ntiles);
   } else {
     auto kern = mlp_fused_kernel<uint16_t>;
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kFLds);
     if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(mlp_fused): %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, grid, dim3(256), kFLds, st, (const uint16_t*)x, (const uint16_t*)w_gated, (const uint16_t*)w_out,
-                       bias, (const uint16_t*)residual, (uint16_t*)out, M, intermediate);
+    hipLaunchKernelGGL(kern, grid, dim3(512), kFLds, st, (const uint16_t*)x, (const unsigned char*)w_packed,
+                       bias, (const uint16_t*)residual, (uint16_t*)out, M, intermediate, ntiles);
   }
   return check_launch("mlp_fused");
 }

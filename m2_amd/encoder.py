@@ -136,13 +136,18 @@ class BertGatedLinearUnitMLP(nn.Module):
     # (d = 768 only).  Off by default: with one wave per SIMD its vector-ALU work (gelu * value) is not hidden behind
     # the MFMAs, and it measured slower on MI355X than the two kernels it replaces (226 against 191 us at M = 32768).
     fuse_mlp = False
+    _packed = None
 
     def presum(self, a16: torch.Tensor) -> torch.Tensor:
         """a16 (M, d) bf16 -> wo(glu(a16)) + bias + a16, (M, d) fp32 (the LayerNorm input)."""
         if self.fuse_mlp and ops.mlp_fused_supported(a16.shape[1], self.config.intermediate_size,
                                                      self.config.monarch_mlp_nblocks):
-            return ops.mlp_fused(a16, self.gated_layers.weight_bf16(), self.wo.weight_bf16(),
-                                 self.wo.bias.detach().float().contiguous(), a16, out_dtype=torch.float32)
+            wg, wo = self.gated_layers.weight_bf16(), self.wo.weight_bf16()
+            # the packed copy the kernel streams: rebuilt whenever one of the bf16 copies has been rebuilt
+            if self._packed is None or self._packed[0] is not wg or self._packed[1] is not wo:
+                self._packed = (wg, wo, ops.mlp_fused_pack(wg, wo))
+            return ops.mlp_fused(a16, wg, wo, self.wo.bias.detach().float().contiguous(), a16, out_dtype=torch.float32,
+                                 packed=self._packed[2])
         g = ops.blockdiag_glu(a16, self.gated_layers.weight_bf16())
         return ops.blockdiag_linear(g, self.wo.weight_bf16(), self.wo.bias.detach().float().contiguous(), a16,
                                     out_dtype=torch.float32)

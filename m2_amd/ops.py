@@ -229,18 +229,36 @@ def mlp_fused_supported(in_features: int, intermediate: int, nblocks: int) -> bo
     return bool(lib.m2_mlp_fused_supported(int(in_features), int(intermediate), int(nblocks)))
 
 
+def mlp_fused_pack(w_gated: Tensor, w_out: Tensor) -> Tensor:
+    """gated_layers.weight (nb, 2I/nb, d/nb) bf16 and wo.weight (nb, d/nb, I/nb) bf16 -> the packed copy `mlp_fused`
+    streams (flat bf16 tensor, as many elements as the two weights together).  Once per set of weights."""
+    nb, q, p = w_gated.shape
+    _require(w_gated, "w_gated", torch.bfloat16)
+    d, I = nb * p, nb * q // 2
+    _require(w_out, "w_out", torch.bfloat16, (nb, d // nb, I // nb))
+    nbytes = int(lib.m2_mlp_fused_packed_bytes(d, I, nb))
+    if nbytes == 0:
+        raise RuntimeError(f"mlp_fused is built for nblocks=4, in_features=768, intermediate % 128 == 0; got {nb}, {d}, {I}")
+    packed = torch.empty(nbytes // 2, dtype=torch.bfloat16, device=w_gated.device)
+    check(lib.m2_mlp_fused_pack(_ptr(w_gated), _ptr(w_out), _ptr(packed), d, I, nb, _stream()))
+    return packed
+
+
 def mlp_fused(x: Tensor, w_gated: Tensor, w_out: Tensor, bias: Optional[Tensor] = None, residual: Optional[Tensor] = None,
-              out_dtype=torch.float32, out: Optional[Tensor] = None) -> Tensor:
+              out_dtype=torch.float32, out: Optional[Tensor] = None, packed: Optional[Tensor] = None) -> Tensor:
     """blockdiag(gelu_erf(h[:, :I]) * h[:, I:], w_out) (+ bias) (+ residual) with h = blockdiag(x, w_gated), one kernel.
-    x (M, d) bf16, w_gated (nb, 2I/nb, d/nb) bf16, w_out (nb, d/nb, I/nb) bf16."""
+    x (M, d) bf16, w_gated (nb, 2I/nb, d/nb) bf16, w_out (nb, d/nb, I/nb) bf16; `packed` = mlp_fused_pack(w_gated,
+    w_out), which a caller with fixed weights computes once (without it the weights are packed on every call)."""
     M, d = x.shape
     nb, q, p = w_gated.shape
     _require(x, "x", torch.bfloat16)
-    _require(w_gated, "w_gated", torch.bfloat16)
     I = nb * q // 2
-    _require(w_out, "w_out", torch.bfloat16, (nb, d // nb, I // nb))
     if nb * p != d:
         raise ValueError(f"x has {d} features, w_gated expects {nb}*{p}")
+    if packed is None:
+        packed = mlp_fused_pack(w_gated, w_out)
+    else:
+        _require(packed, "packed", torch.bfloat16, (int(lib.m2_mlp_fused_packed_bytes(d, I, nb)) // 2,))
     if bias is not None:
         _require(bias, "bias", torch.float32, (d,))
     if residual is not None:
@@ -249,7 +267,7 @@ def mlp_fused(x: Tensor, w_gated: Tensor, w_out: Tensor, bias: Optional[Tensor] 
         out = torch.empty(M, d, dtype=out_dtype, device=x.device)
     else:
         _require(out, "out", out_dtype, (M, d))
-    check(lib.m2_mlp_fused_fwd(_ptr(x), _ptr(w_gated), _ptr(w_out), _ptr(bias), _ptr(residual), _ptr(out), M, d, I, nb,
+    check(lib.m2_mlp_fused_fwd(_ptr(x), _ptr(packed), _ptr(bias), _ptr(residual), _ptr(out), M, d, I, nb,
                                _act_code(out_dtype), _stream()))
     return out
 
