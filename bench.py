@@ -272,6 +272,7 @@ def main():
     for fn, tag in (("mixer_core", "mixer_core"), ("hyena_filter_taps", "filter_taps"),
                     ("filter_spectrum", "filter_spectrum"), ("blockdiag_glu", "blockdiag_glu"),
                     ("blockdiag_linear", "blockdiag_linear"), ("blockdiag_linear_layernorm", "wo_layernorm"),
+                    ("mlp_fused", "mlp_fused"),
                     ("layernorm", "layernorm"), ("embed_layernorm", "embed_layernorm")):
         wrapped[fn] = timer.wrap(ops, fn, tag)
 
@@ -288,7 +289,8 @@ def main():
         dt = time.perf_counter() - t0
     eager_ms = dt / args.steps * 1e3
     means = {tag: timer.mean_ms(tag) for tag in ("mixer_core", "filter_taps", "filter_spectrum", "blockdiag_glu",
-                                                  "blockdiag_linear", "wo_layernorm", "layernorm", "embed_layernorm")
+                                                  "blockdiag_linear", "wo_layernorm", "mlp_fused", "layernorm",
+                                                  "embed_layernorm")
              if timer.count(tag)}
     n_core = timer.count("mixer_core")
     for fn, orig in wrapped.items():            # per-launch events are only wanted for the eager timed steps
@@ -343,27 +345,37 @@ def main():
     nbk = cfg.monarch_mlp_nblocks
     glu_flops = 2 * M * d * 2 * I / nbk
     wo_flops = 2 * M * I * d / nbk
-    t_glu = means["blockdiag_glu"]
-    # the same kernels against the HBM roof: algorithmic bytes (bf16 in, fused GLU write; wo with its bf16 residual
-    # and fp32 sum) over the measured time, as a fraction of 8 TB/s
-    glu_bytes = M * d * 2 + (2 * I * d // nbk) * 2 + M * I * 2
-    wo_bytes = M * I * 2 + (I * d // nbk) * 2 + M * d * 2 + M * d * 4
-    glu_tflops = glu_flops / (t_glu * 1e-3) / 1e12
-    k3 = {"kernel": "gated block-diagonal GEMM + GLU (m2_blockdiag_glu_fwd)", "bound": "mfma", "achieved": glu_tflops,
-          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": glu_tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-          "flops_per_launch": glu_flops, "ms_per_launch": t_glu,
-          "hbm_frac": glu_bytes / (t_glu * 1e-3) / 1e9 / HBM_PEAK_GBPS}
-    if "wo_layernorm" in means:        # wo + bias + residual + LayerNorm as one kernel (an option, d <= 768)
-        t_wo = means["wo_layernorm"]
-        k3["wo_kernel"] = "wo + bias + residual + LayerNorm (m2_blockdiag_linear_layernorm_fwd)"
+    if "mlp_fused" in means:           # the whole MLP as one kernel (d = 768): the (M, I) intermediate never reaches HBM
+        t_mlp = means["mlp_fused"]
+        mlp_bytes = M * d * 2 + (3 * I * d // nbk) * 2 + M * d * 2 + M * d * 4
+        mlp_tflops = (glu_flops + wo_flops) / (t_mlp * 1e-3) / 1e12
+        k3 = {"kernel": "gated block-diagonal GEMM + GLU + wo + bias + residual as one kernel (m2_mlp_fused_fwd)",
+              "bound": "mfma", "achieved": mlp_tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+              "frac": mlp_tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "flops_per_launch": glu_flops + wo_flops,
+              "ms_per_launch": t_mlp, "hbm_frac": mlp_bytes / (t_mlp * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+              "both_frac": mlp_tflops / MFMA_BF16_PEAK_TFLOPS}
     else:
-        t_wo = means["blockdiag_linear"]
-        k3["wo_kernel"] = "wo + bias + residual (m2_blockdiag_linear_fwd)"
-        k3["wo_hbm_frac"] = wo_bytes / (t_wo * 1e-3) / 1e9 / HBM_PEAK_GBPS
-    k3["wo_achieved"] = wo_flops / (t_wo * 1e-3) / 1e12
-    k3["wo_frac"] = k3["wo_achieved"] / MFMA_BF16_PEAK_TFLOPS
-    k3["wo_ms_per_launch"] = t_wo
-    k3["both_frac"] = (glu_flops + wo_flops) / ((t_glu + t_wo) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
+        t_glu = means["blockdiag_glu"]
+        # the same kernels against the HBM roof: algorithmic bytes (bf16 in, fused GLU write; wo with its bf16
+        # residual and fp32 sum) over the measured time, as a fraction of 8 TB/s
+        glu_bytes = M * d * 2 + (2 * I * d // nbk) * 2 + M * I * 2
+        wo_bytes = M * I * 2 + (I * d // nbk) * 2 + M * d * 2 + M * d * 4
+        glu_tflops = glu_flops / (t_glu * 1e-3) / 1e12
+        k3 = {"kernel": "gated block-diagonal GEMM + GLU (m2_blockdiag_glu_fwd)", "bound": "mfma", "achieved": glu_tflops,
+              "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": glu_tflops / MFMA_BF16_PEAK_TFLOPS,
+              "traffic": None, "flops_per_launch": glu_flops, "ms_per_launch": t_glu,
+              "hbm_frac": glu_bytes / (t_glu * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        if "wo_layernorm" in means:        # wo + bias + residual + LayerNorm as one kernel (an option, d <= 768)
+            t_wo = means["wo_layernorm"]
+            k3["wo_kernel"] = "wo + bias + residual + LayerNorm (m2_blockdiag_linear_layernorm_fwd)"
+        else:
+            t_wo = means["blockdiag_linear"]
+            k3["wo_kernel"] = "wo + bias + residual (m2_blockdiag_linear_fwd)"
+            k3["wo_hbm_frac"] = wo_bytes / (t_wo * 1e-3) / 1e9 / HBM_PEAK_GBPS
+        k3["wo_achieved"] = wo_flops / (t_wo * 1e-3) / 1e12
+        k3["wo_frac"] = k3["wo_achieved"] / MFMA_BF16_PEAK_TFLOPS
+        k3["wo_ms_per_launch"] = t_wo
+        k3["both_frac"] = (glu_flops + wo_flops) / ((t_glu + t_wo) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
 
     result = {
         "metric": "seq/s M2-BERT-80M fwd at L=8192; FFT-conv HBM GB/s & % of peak" if args.config == "c3"

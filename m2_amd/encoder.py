@@ -133,9 +133,10 @@ class BertGatedLinearUnitMLP(nn.Module):
     # L = 8192, B = 4; 2.00 against 2.24 ms at L = 128, B = 32), although it writes and re-reads the fp32 sum.
     fuse_wo_layernorm = False
     # True: gated_layers, GLU and wo + bias + residual as one kernel that keeps the (M, I) intermediate on chip
-    # (d = 768 only).  Off by default: with one wave per SIMD its vector-ALU work (gelu * value) is not hidden behind
-    # the MFMAs, and it measured slower on MI355X than the two kernels it replaces (226 against 191 us at M = 32768).
-    fuse_mlp = False
+    # (d = 768, four blocks; other shapes take the two kernels).  Measured on MI355X at M = 32768: 175 - 183 us against
+    # 191 us for the two kernels it replaces.  It streams the weights from a packed copy (3.5 MB per layer at
+    # I = 3072) that is rebuilt when the weights change.
+    fuse_mlp = True
     _packed = None
 
     def presum(self, a16: torch.Tensor) -> torch.Tensor:
