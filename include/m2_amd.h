@@ -61,7 +61,9 @@ typedef struct m2_hyena_filter_params {
   const float* rw3;
 } m2_hyena_filter_params;
 
-/* Bytes of fp32 workspace m2_hyena_filter_fwd needs for `nfilters` filters of length L. */
+/* Bytes of workspace m2_hyena_filter_fwd needs for `nfilters` filters of length L: the last hidden layer's
+ * activations (2 nfilters L order fp32-sized values) and the inner-layer weights re-split for the matrix cores
+ * (2 nfilters x 2 layers x 3 bf16 parts x order^2). */
 size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int order);
 
 /* taps[f] (d, 2L) fp32, f < nfilters:  taps[f][c][l]      = k_fwd[c][l]       for l < L
@@ -82,7 +84,7 @@ int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int 
  * the array: two such calls whose kernels may overlap on the same GPU (different streams, or different host threads
  * on different streams) race; calls on one stream are ordered and safe.  The first call on a device looks up the
  * array's device address (hipGetSymbolAddress): make that call outside a stream capture. */
-#define M2_HYENA_FILTER_STATIC_SCRATCH_BYTES (16u << 20)
+#define M2_HYENA_FILTER_STATIC_SCRATCH_BYTES (17u << 20)
 int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order,
                                int emb_dim, float w_mod, float shift, float* taps, void* stream);
 

@@ -232,9 +232,16 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_split_kernel(
                        scale * (zb.re - za.re));
   };
 
-  // work item = (channel, half transform): 2 d items spread evenly over the grid
-  for (int item = blockIdx.x; item < 2 * d; item += gridDim.x) {
-    const int c = item >> 1;
+  // work item = (channel, half transform): 2 d items spread evenly over the grid.  Workgroup ids are dealt round-robin
+  // to the 8 XCDs (one L2 each): XCD e takes the channels c = e (mod 8), and the two halves of a channel, which read the
+  // same taps, run on neighbouring workgroups of that XCD at the same time, so the second read is an L2 hit.
+  // (Needs d % 8 == 0 and an even number of workgroups per XCD; other shapes take the items in plain order.)
+  const bool by_xcd = (d & 7) == 0 && (gridDim.x & 15) == 0;
+  const int first = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x, step = by_xcd ? (int)(gridDim.x >> 3) : (int)gridDim.x;
+  const int count = by_xcd ? (d >> 3) * 2 : 2 * d;
+  for (int j = first; j < count; j += step) {
+    const int c = by_xcd ? (j >> 1) * 8 + (int)(blockIdx.x & 7) : j >> 1;
+    const int item = j;
     auto one_half = [&](auto hh) __attribute__((always_inline)) {
       constexpr bool ODD = decltype(hh)::value == 1;
       // z = k1 + i k2 over 2L taps; even half: z_lo + z_hi, odd half: z_lo - z_hi (its twist is in the first pass).
@@ -342,7 +349,8 @@ static int launch_filter_spectrum_split_t(const float* taps1, const float* taps2
   int per_cu = (int)((160 * 1024) / lds_bytes);
   if (per_cu < 1) per_cu = 1;
   if (per_cu > 512 / P::T) per_cu = 512 / P::T;
-  int grid = num_cus() * per_cu;
+  // a multiple of 16 workgroups: an even number per XCD, so that the two halves of a channel run side by side
+  int grid = (num_cus() * per_cu) / 16 * 16;
   if (grid > 2 * d) grid = 2 * d;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(P::T), lds_bytes, stream, taps1, taps2, D1, D2, (float4*)spec, d);
   return check_launch("filter_spectrum_split");

@@ -6,18 +6,21 @@
 // (bert/src/mm/hyena_utils.py:168-175 the MLP, :50-63 Sin, :110-112 modulation, :201-217 filter /
 // filter_rev, :231-236 placement of the forward and the flipped reverse taps in a 2L window.)
 //
-// Two kernels.  `hidden_kernel` evaluates the three sin layers for a tile of 32 positions: the first
-// (emb -> 128) on the vector ALU, the two 128 x 128 layers as fp32 MFMA GEMMs
-// (v_mfma_f32_32x32x2_f32: exact fp32 products, which matters because sin(freq * x) amplifies any
-// rounding of x) with the activations resident in LDS; it writes h3 split into a bf16 high part and
-// a bf16 low part (h3 = hi + lo to 16 mantissa bits).  `project_kernel` is the 128 -> d projection as
-// a three-product split-bf16 MFMA GEMM (W_hi h_hi + W_hi h_lo + W_lo h_hi, v_mfma_f32_32x32x16_bf16,
-// fp32 accumulate; 4.6e-6 relative error against fp64, measured) whose epilogue applies the decay and
-// stores the taps channel-major, forward taps at [0, L) and reverse taps mirrored into [L, 2L).
+// Three kernels.  `split_weights_kernel` re-splits the 128 x 128 weights of the two inner layers into three bf16
+// parts in MFMA operand layout (a few microseconds, once per call).  `hidden_kernel` evaluates the three sin layers
+// for 32 - 128 positions per workgroup: the first (emb -> 128) on the vector ALU, the two 128 x 128 layers as
+// six-product split-bf16 MFMA GEMMs (v_mfma_f32_32x32x16_bf16 on the three parts of weights and activations: all
+// product terms down to 2^-24, i.e. fp32 products, which matters because sin(freq * x) amplifies any rounding of
+// x) with the activations resident in LDS; it writes h3 split into a bf16 high part and a bf16 low part
+// (h3 = hi + lo to 16 mantissa bits).  `project_kernel` is the 128 -> d projection as a three-product split-bf16
+// MFMA GEMM (W_hi h_hi + W_hi h_lo + W_lo h_hi, fp32 accumulate; 4.6e-6 relative error against fp64, measured)
+// whose epilogue applies the decay and stores the taps channel-major, forward taps at [0, L) and reverse taps
+// mirrored into [L, 2L).
 #include <hip/hip_runtime.h>
 
 #include <mutex>
 
+#include "fft_regs.h"
 #include "m2_internal.h"
 
 namespace m2 {
@@ -60,78 +63,164 @@ __device__ __forceinline__ float sin_reduced(float x) {
   return (static_cast<int>(n) & 1) ? -s : s;
 }
 
-constexpr int kActRow = kOrder + 4;       // padded fp32 row of the activation tile (bank-conflict-free b128 reads)
+__device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  u32x4 v = {a, b, c, d};
+  return __builtin_bit_cast(bf16x8, v);
+}
 
-// grid (L / 32, 2 * nfilters), block 256 = 4 waves; wave w owns output neurons [32 w, 32 w + 32).
+// x = hi + mid + lo with three bf16 terms: 24 mantissa bits, i.e. all of an fp32 value
+__device__ __forceinline__ void split3(float x, float& hi, float& mid, float& lo) {
+  hi = bf16_to_f32(f32_to_bf16(x));
+  const float r = x - hi;
+  mid = bf16_to_f32(f32_to_bf16(r));
+  lo = r - mid;                      // the conversion of lo to bf16 happens where it is packed
+}
+
+// The 128 x 128 weights of the two inner layers, split into three bf16 parts and laid out as MFMA A operands, so
+// that hidden_kernel fetches them with coalesced 16-byte loads and no arithmetic:
+// wsplit[mlp][layer][part][wave w][K step ks][lane (i, h)] = 8 bf16 of row 32 w + i, K = 16 ks + 8 h .. + 7.
+constexpr int kSplitPerLayer = 3 * kOrder * kOrder;      // bf16 elements per (mlp, layer)
+__global__ __launch_bounds__(256) void split_weights_kernel(FilterBatch fb, int nmlp, uint16_t* __restrict__ wsplit) {
+  const int id = blockIdx.x * 256 + threadIdx.x;             // (mlp, layer, wave, ks, lane)
+  const int lane = id & 63, ks = (id >> 6) & 7, w = (id >> 9) & 3, layer = (id >> 11) & 1, m = id >> 12;
+  if (m >= nmlp) return;
+  const MlpPtrs& W = fb.f[m >> 1].mlp[m & 1];
+  if (W.w0 == nullptr) return;
+  const float* src = (layer == 0 ? W.w1 : W.w2) + (long)(32 * w + (lane & 31)) * kOrder + 16 * ks + 8 * (lane >> 5);
+  float h[8], md[8], l[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) split3(src[j], h[j], md[j], l[j]);
+  u32x4* dst = reinterpret_cast<u32x4*>(wsplit + ((long)(m * 2 + layer)) * kSplitPerLayer) + (w * 8 + ks) * 64 + lane;
+  const u32x4 vh = {pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]), pack_bf16x2(h[4], h[5]), pack_bf16x2(h[6], h[7])};
+  const u32x4 vm = {pack_bf16x2(md[0], md[1]), pack_bf16x2(md[2], md[3]), pack_bf16x2(md[4], md[5]), pack_bf16x2(md[6], md[7])};
+  const u32x4 vl = {pack_bf16x2(l[0], l[1]), pack_bf16x2(l[2], l[3]), pack_bf16x2(l[4], l[5]), pack_bf16x2(l[6], l[7])};
+  dst[0] = vh;
+  dst[kOrder * kOrder / 8] = vm;
+  dst[2 * kOrder * kOrder / 8] = vl;
+}
+
+constexpr int kActRowB = 2 * kOrder + 16;     // bytes per padded bf16 row of an activation part (conflict-free 16-byte reads)
+
+// grid (L / (32 TILES), 2 * nfilters), block 256 = 4 waves.  Wave w owns the output neurons [32 w, 32 w + 32) of all
+// TILES tiles of 32 positions of the workgroup.  The activations live in LDS as three bf16 parts (hi, mid, lo:
+// together the fp32 value) and every layer overwrites them in place; the two 128 x 128 layers are six-product
+// split-bf16 MFMA GEMMs (all products of the three parts of either operand down to 2^-24 relative: fp32 accuracy,
+// which matters because sin(freq * x) amplifies any rounding of x, at 2.7 times the rate of fp32 MFMAs), their
+// weights pre-split by split_weights_kernel and held in registers for all tiles (fetching them is what a short run
+// of positions per workgroup pays most for: 96 KB per workgroup and layer from L2).  Within a layer the products of
+// tile i + 1 are issued together with the sin epilogue of tile i, so that matrix pipe and vector ALU overlap.
+template <int TILES>
 __global__ __launch_bounds__(256) void hidden_kernel(FilterBatch fb, int L, int emb, float w_mod,
+                                                     const uint16_t* __restrict__ wsplit,
                                                      uint16_t* __restrict__ h_hi /* (2 nf, L, 128) bf16 */,
                                                      uint16_t* __restrict__ h_lo /* (2 nf, L, 128) bf16 */) {
-  __shared__ __attribute__((aligned(16))) float act[2][kPosTile][kActRow];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
+  constexpr int P = 32 * TILES;
+  __shared__ __attribute__((aligned(16))) unsigned char act[3][P * kActRowB];
+  __shared__ float zt[P * kMaxEmb];
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
   const int fi = blockIdx.y >> 1, dir = blockIdx.y & 1;
   const FilterPtrs& F = fb.f[fi];
   const MlpPtrs& W = F.mlp[dir];
   if (W.w0 == nullptr) return;                  // not bidirectional: nothing to do for dir == 1
-  const int l0 = blockIdx.x * kPosTile;
+  const int l0 = blockIdx.x * P;
 
-  // layer 0 (emb -> 128) on the vector ALU: thread = (neuron o, 16 positions).  The tile's embeddings
-  // (32 x emb consecutive floats) go through LDS; weights beyond emb are zero so the dot product has a
-  // fixed length.
+  auto put3 = [&](int pos, int o, float v0, float v1, float v2, float v3) __attribute__((always_inline)) {
+    float h[4], m[4], l[4];
+    split3(v0, h[0], m[0], l[0]); split3(v1, h[1], m[1], l[1]); split3(v2, h[2], m[2], l[2]); split3(v3, h[3], m[3], l[3]);
+    const int off = pos * kActRowB + 2 * o;
+    *reinterpret_cast<uint2*>(&act[0][off]) = make_uint2(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]));
+    *reinterpret_cast<uint2*>(&act[1][off]) = make_uint2(pack_bf16x2(m[0], m[1]), pack_bf16x2(m[2], m[3]));
+    *reinterpret_cast<uint2*>(&act[2][off]) = make_uint2(pack_bf16x2(l[0], l[1]), pack_bf16x2(l[2], l[3]));
+  };
+
+  // Weights of an inner layer -> registers.  Requested one phase early (layer 1's before the vector-ALU layer, layer
+  // 2's before the last epilogue of layer 1), so that the 24 KB per wave arrive behind other work.
+  bf16x8 ah[8], am[8], al[8];
+  auto load_weights = [&](int layer) __attribute__((always_inline)) {
+    const u32x4* wp = reinterpret_cast<const u32x4*>(wsplit + ((long)(blockIdx.y * 2 + layer)) * kSplitPerLayer) + w * 8 * 64 + lane;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      ah[ks] = __builtin_bit_cast(bf16x8, wp[ks * 64]);
+      am[ks] = __builtin_bit_cast(bf16x8, wp[ks * 64 + kOrder * kOrder / 8]);
+      al[ks] = __builtin_bit_cast(bf16x8, wp[ks * 64 + 2 * kOrder * kOrder / 8]);
+    }
+  };
+  load_weights(0);
+
+  // layer 0 (emb -> 128) on the vector ALU: thread = (4 neurons, P / 8 positions).  The embeddings of the tile
+  // (P x emb consecutive floats) go through LDS; weights beyond emb are zero so the dot product has a fixed length.
   {
-    __shared__ float zt[kPosTile * kMaxEmb];
-    zt[tid] = tid < kPosTile * emb ? F.z[(long)l0 * emb + tid] : 0.f;
-    const int o = tid & (kOrder - 1), p0 = (tid >> 7) * 16;
-    float w[kMaxEmb];
+    for (int i = tid; i < P * kMaxEmb; i += 256) zt[i] = i < P * emb ? F.z[(long)l0 * emb + i] : 0.f;
+    const int o = 4 * (tid & 31), p0 = tid >> 5;          // positions p0, p0 + 8, ...
+    float wt[4][kMaxEmb], bb[4], fo[4];
 #pragma unroll
-    for (int e = 0; e < kMaxEmb; ++e) w[e] = e < emb ? W.w0[o * emb + e] : 0.f;
-    const float b = W.b0[o], fo = w_mod * F.freq[o];
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int e = 0; e < kMaxEmb; ++e) wt[j][e] = e < emb ? W.w0[(o + j) * emb + e] : 0.f;
+      bb[j] = W.b0[o + j];
+      fo[j] = w_mod * F.freq[o + j];
+    }
     __syncthreads();
-#pragma unroll
-    for (int pp = 0; pp < 16; ++pp) {
-      const int p = p0 + pp;
-      const int zi = p * emb;
-      float acc = b;
-#pragma unroll
-      for (int e = 0; e < kMaxEmb; ++e) acc += w[e] * zt[zi + e];      // zi + e <= 31 emb + 7 < 256
-      act[0][p][o] = sin_reduced(fo * acc);
-    }
-  }
-  __syncthreads();
-  // layers 1, 2: D[o'][pos] = sum_o W[o'][o] act[pos][o].  Lane (i32, half) holds K = 8 q + 4 half + {0..3}
-  // of weight row 32 wave + i32 and of position i32: four MFMA steps per pair of float4.
-  for (int layer = 0; layer < 2; ++layer) {
-    const float* wm = (layer == 0 ? W.w1 : W.w2) + (long)(32 * wave + i32) * kOrder + 4 * half;
-    const float* bias = layer == 0 ? W.b1 : W.b2;
-    const int src = layer & 1, dst = src ^ 1;
-    float4 av[kOrder / 8];
-#pragma unroll
-    for (int q = 0; q < kOrder / 8; ++q) av[q] = *reinterpret_cast<const float4*>(wm + 8 * q);
-    const float* bp = &act[src][i32][4 * half];
-    floatx16 acc;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-#pragma unroll
-    for (int q = 0; q < kOrder / 8; ++q) {
-      const float4 bv = *reinterpret_cast<const float4*>(bp + 8 * q);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].x, bv.x, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].y, bv.y, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].z, bv.z, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].w, bv.w, acc, 0, 0, 0);
-    }
-    // accumulator element v: neuron 32 wave + 8 (v / 4) + 4 half + v % 4, position i32
-    const long hrow = ((long)blockIdx.y * L + l0 + i32) * kOrder;
-#pragma unroll
-    for (int vq = 0; vq < 4; ++vq) {
-      const int o = 32 * wave + 8 * vq + 4 * half;
-      const float4 fq = *reinterpret_cast<const float4*>(F.freq + o);
-      const float4 bq = *reinterpret_cast<const float4*>(bias + o);
-      const float fr[4] = {fq.x, fq.y, fq.z, fq.w}, bs[4] = {bq.x, bq.y, bq.z, bq.w};
+#pragma unroll 4
+    for (int pp = 0; pp < P / 8; ++pp) {
+      const int pos = p0 + 8 * pp;
       float s[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s[j] = sin_reduced(w_mod * fr[j] * (acc[4 * vq + j] + bs[j]));
-      if (layer == 0) {
-        *reinterpret_cast<float4*>(&act[dst][i32][o]) = make_float4(s[0], s[1], s[2], s[3]);
+      for (int j = 0; j < 4; ++j) {
+        float acc = bb[j];
+#pragma unroll
+        for (int e = 0; e < kMaxEmb; ++e) acc += wt[j][e] * zt[pos * emb + e];      // pos emb + e < P emb + 8 <= P kMaxEmb
+        s[j] = sin_reduced(fo[j] * acc);
+      }
+      put3(pos, o, s[0], s[1], s[2], s[3]);
+    }
+  }
+  // layers 1, 2: D[o'][pos] = sum_o W[o'][o] act[pos][o].  A = weight rows 32 w + i32 (registers), B = positions of the
+  // tile (LDS); lane (i32, half) holds K = 16 ks + 8 half .. + 7 of both.
+  auto products = [&](int tile, floatx16& acc) __attribute__((always_inline)) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+    const int boff = (32 * tile + i32) * kActRowB + 16 * half;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const bf16x8 bh = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&act[0][boff + 32 * ks]));
+      const bf16x8 bm = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&act[1][boff + 32 * ks]));
+      const bf16x8 bl = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&act[2][boff + 32 * ks]));
+      // smallest terms first
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[ks], bh, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bl, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am[ks], bm, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am[ks], bh, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bm, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bh, acc, 0, 0, 0);
+    }
+  };
+  // accumulator element v: neuron 32 w + 8 (v / 4) + 4 half + v % 4, position i32 of the tile
+  float fr[16], bs[16];
+  auto load_scales = [&](int layer) __attribute__((always_inline)) {
+    const float* bias = layer == 0 ? W.b1 : W.b2;
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq) {
+      const int o = 32 * w + 8 * vq + 4 * half;
+      const float4 fq = *reinterpret_cast<const float4*>(F.freq + o);
+      const float4 bq = *reinterpret_cast<const float4*>(bias + o);
+      fr[4 * vq] = w_mod * fq.x; fr[4 * vq + 1] = w_mod * fq.y; fr[4 * vq + 2] = w_mod * fq.z; fr[4 * vq + 3] = w_mod * fq.w;
+      bs[4 * vq] = bq.x; bs[4 * vq + 1] = bq.y; bs[4 * vq + 2] = bq.z; bs[4 * vq + 3] = bq.w;
+    }
+  };
+  auto epilogue = [&](auto ll, int tile, const floatx16& acc) __attribute__((always_inline)) {
+    constexpr int layer = decltype(ll)::value;
+    const int pos = 32 * tile + i32;
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq) {
+      const int o = 32 * w + 8 * vq + 4 * half;
+      float s[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[j] = sin_reduced(fr[4 * vq + j] * (acc[4 * vq + j] + bs[4 * vq + j]));
+      if constexpr (layer == 0) {
+        put3(pos, o, s[0], s[1], s[2], s[3]);
       } else {
+        const long hrow = ((long)blockIdx.y * L + l0 + pos) * kOrder;
         float hi[4], lo[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -142,13 +231,28 @@ __global__ __launch_bounds__(256) void hidden_kernel(FilterBatch fb, int L, int 
         *reinterpret_cast<uint2*>(h_lo + hrow + o) = make_uint2(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]));
       }
     }
+  };
+  // One layer: products(0); then for every tile "barrier; products(next tile) with epilogue(this tile)".  The barrier
+  // before an epilogue says that all four waves have read that tile's operands, so it may be overwritten in place;
+  // the barrier that ends the layer says that all of the layer's activations are written.
+  auto layer_pass = [&](auto ll) __attribute__((always_inline)) {
+    constexpr int layer = decltype(ll)::value;
+    floatx16 acc[2];
+    products(0, acc[0]);
+    static_for<0, TILES>([&](auto tt) {
+      constexpr int t = decltype(tt)::value;
+      __syncthreads();
+      if constexpr (t + 1 < TILES) products(t + 1, acc[(t + 1) & 1]);
+      else if constexpr (layer == 0) load_weights(1);      // the products of layer 1 are done: its registers are free
+      epilogue(ll, t, acc[t & 1]);
+    });
     __syncthreads();
-  }
-}
-
-__device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
-  u32x4 v = {a, b, c, d};
-  return __builtin_bit_cast(bf16x8, v);
+  };
+  load_scales(0);
+  __syncthreads();                     // layer 0's activations are complete
+  layer_pass(ic<0>{});
+  load_scales(1);
+  layer_pass(ic<1>{});
 }
 
 // Workgroup = 4 waves = 128 channels; wave w owns channels [c0 + 32 w, + 32) with its weight rows split
@@ -185,20 +289,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
   const uint16_t* gh = h_hi + ((long)blockIdx.z * L + lbase) * kOrder + 8 * tid;
   const uint16_t* gl = h_lo + ((long)blockIdx.z * L + lbase) * kOrder + 8 * tid;
   const int srow0 = tid >> 4, scol = (tid & 15) * 16;              // piece q covers row srow0 + 16 q
-  u32x4 st[4];
-  auto fetch = [&](int pt) __attribute__((always_inline)) {
-    st[0] = *reinterpret_cast<const u32x4*>(gh + pt * tile_elems);
-    st[1] = *reinterpret_cast<const u32x4*>(gh + pt * tile_elems + 16 * kOrder);
-    st[2] = *reinterpret_cast<const u32x4*>(gl + pt * tile_elems);
-    st[3] = *reinterpret_cast<const u32x4*>(gl + pt * tile_elems + 16 * kOrder);
+  // two register sets: the tile after next is in flight while the next one waits to be staged (a tile's product
+  // takes well under a memory latency, so one tile of look-ahead left every iteration waiting for its fetch)
+  u32x4 st[2][4];
+  auto fetch = [&](int pt, auto ss) __attribute__((always_inline)) {
+    constexpr int s = decltype(ss)::value;
+    st[s][0] = *reinterpret_cast<const u32x4*>(gh + pt * tile_elems);
+    st[s][1] = *reinterpret_cast<const u32x4*>(gh + pt * tile_elems + 16 * kOrder);
+    st[s][2] = *reinterpret_cast<const u32x4*>(gl + pt * tile_elems);
+    st[s][3] = *reinterpret_cast<const u32x4*>(gl + pt * tile_elems + 16 * kOrder);
   };
-  auto stage = [&](int buf) __attribute__((always_inline)) {
-    *reinterpret_cast<u32x4*>(&hbuf[buf][0][srow0 * kHRow + scol]) = st[0];
-    *reinterpret_cast<u32x4*>(&hbuf[buf][0][(srow0 + 16) * kHRow + scol]) = st[1];
-    *reinterpret_cast<u32x4*>(&hbuf[buf][1][srow0 * kHRow + scol]) = st[2];
-    *reinterpret_cast<u32x4*>(&hbuf[buf][1][(srow0 + 16) * kHRow + scol]) = st[3];
+  auto stage = [&](int buf, auto ss) __attribute__((always_inline)) {
+    constexpr int s = decltype(ss)::value;
+    *reinterpret_cast<u32x4*>(&hbuf[buf][0][srow0 * kHRow + scol]) = st[s][0];
+    *reinterpret_cast<u32x4*>(&hbuf[buf][0][(srow0 + 16) * kHRow + scol]) = st[s][1];
+    *reinterpret_cast<u32x4*>(&hbuf[buf][1][srow0 * kHRow + scol]) = st[s][2];
+    *reinterpret_cast<u32x4*>(&hbuf[buf][1][(srow0 + 16) * kHRow + scol]) = st[s][3];
   };
-  fetch(0);
+  fetch(0, ic<0>{});
+  if (ntiles > 1) fetch(1, ic<1>{});
 
   // A operand: rows c0 + i32, K = 16 ks + 8 half + {0..7}, split hi / lo
   bf16x8 ahi[kOrder / 16], alo[kOrder / 16];
@@ -222,14 +331,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
 #pragma unroll
     for (int v = 0; v < 16; ++v) adelta[v] = -fabsf(F.deltas[c0 + 8 * (v >> 2) + 4 * half + (v & 3)]) * 1.44269504088896341f;
   }
-  stage(0);
+  stage(0, ic<0>{});
   __syncthreads();
 
-  for (int pt = 0; pt < ntiles; ++pt) {
-    if (pt + 1 < ntiles) fetch(pt + 1);
+  // iteration pt: tile pt is in hbuf[pt & 1], tile pt + 1 in register set (pt + 1) & 1; tile pt + 2 is requested into
+  // the set tile pt was staged from
+  auto iteration = [&](int pt, auto par) __attribute__((always_inline)) {
+    constexpr int P = decltype(par)::value;      // pt & 1
+    if (pt + 2 < ntiles) fetch(pt + 2, ic<P>{});
     if (active) {
-      const unsigned char* bh = &hbuf[pt & 1][0][i32 * kHRow + 16 * half];
-      const unsigned char* bl = &hbuf[pt & 1][1][i32 * kHRow + 16 * half];
+      const unsigned char* bh = &hbuf[P][0][i32 * kHRow + 16 * half];
+      const unsigned char* bl = &hbuf[P][1][i32 * kHRow + 16 * half];
       floatx16 acc;
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[v] = 0.f;
@@ -253,8 +365,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
         po[(long)(8 * (v >> 2) + (v & 3)) * 2 * L] = acc[v] * decay;
       }
     }
-    if (pt + 1 < ntiles) stage((pt + 1) & 1);
+    if (pt + 1 < ntiles) stage(P ^ 1, ic<P ^ 1>{});
     __syncthreads();
+  };
+  for (int pt = 0; pt < ntiles; pt += 2) {
+    iteration(pt, ic<0>{});
+    if (pt + 1 < ntiles) iteration(pt + 1, ic<1>{});
   }
 }
 
@@ -264,7 +380,8 @@ using namespace m2;
 
 extern "C" size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int order) {
   if (nfilters <= 0 || L <= 0 || order <= 0) return 0;
-  return (size_t)2 * nfilters * L * order * sizeof(float);
+  // h3 as bf16 hi / lo parts, then the inner-layer weights of the 2 nfilters MLPs as three bf16 parts each
+  return (size_t)2 * nfilters * L * order * sizeof(float) + (size_t)2 * nfilters * 2 * 3 * order * order * sizeof(uint16_t);
 }
 
 // Shared by the two entry points: validation and the two launches, `workspace` holding the h3 hi / lo parts.
@@ -295,8 +412,17 @@ static int hyena_filter_launch(const char* who, const m2_hyena_filter_params* pa
   hipStream_t s = (hipStream_t)stream;
   uint16_t* h_hi = reinterpret_cast<uint16_t*>(workspace);
   uint16_t* h_lo = h_hi + (size_t)2 * nfilters * L * order;
-  hipLaunchKernelGGL(hidden_kernel, dim3(L / kPosTile, 2 * nfilters), dim3(256), 0, s, fb, L, emb_dim, w_mod, h_hi, h_lo);
-  int rc = check_launch("hyena hidden_kernel");
+  uint16_t* wsplit = h_lo + (size_t)2 * nfilters * L * order;
+  hipLaunchKernelGGL(split_weights_kernel, dim3(2 * nfilters * 2 * 4 * 8 * 64 / 256), dim3(256), 0, s, fb, 2 * nfilters, wsplit);
+  int rc = check_launch("hyena split_weights_kernel");
+  if (rc) return rc;
+  // positions per workgroup: longer runs amortise the weight fetch (96 KB per workgroup and layer), short sequences
+  // need the workgroups spread over the chip
+  if (L % 64 == 0 && L >= 1024)      // measured at L = 8192: 26.9 us with two tiles, 29.5 with four, 32.7 with one
+    hipLaunchKernelGGL(hidden_kernel<2>, dim3(L / 64, 2 * nfilters), dim3(256), 0, s, fb, L, emb_dim, w_mod, wsplit, h_hi, h_lo);
+  else
+    hipLaunchKernelGGL(hidden_kernel<1>, dim3(L / 32, 2 * nfilters), dim3(256), 0, s, fb, L, emb_dim, w_mod, wsplit, h_hi, h_lo);
+  rc = check_launch("hyena hidden_kernel");
   if (rc) return rc;
   hipLaunchKernelGGL(project_kernel, dim3((L + kPosPerWg - 1) / kPosPerWg, (d + 127) / 128, 2 * nfilters), dim3(256), 0, s, fb, L, d, shift,
                      h_hi, h_lo, taps);
@@ -361,8 +487,8 @@ extern "C" int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, 
   void* ptr = nullptr;
   int rc = static_scratch_for_current_device(&ptr);
   if (rc) return rc;
-  // hidden_kernel writes every h3 element project_kernel reads in the same call, so nothing left by an earlier
-  // (possibly longer) call is ever read and nothing needs clearing
+  // split_weights_kernel and hidden_kernel write every element the later kernels of the same call read, so nothing
+  // left by an earlier (possibly longer) call is ever read and nothing needs clearing
   return hyena_filter_launch("m2_hyena_filter_fwd_static", params, nfilters, L, d, order, emb_dim, w_mod, shift, ptr,
                              taps, stream);
 }
