@@ -61,10 +61,10 @@ typedef struct m2_hyena_filter_params {
   const float* rw3;
 } m2_hyena_filter_params;
 
-/* Bytes of workspace m2_hyena_filter_fwd needs for `nfilters` filters of length L: the last hidden layer's
- * activations (2 nfilters L order fp32-sized values) and the inner-layer weights re-split for the matrix cores
- * (2 nfilters x 2 layers x 3 bf16 parts x order^2). */
-size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int order);
+/* Bytes of workspace m2_hyena_filter_fwd needs for `nfilters` filters of length L and width d: the last hidden
+ * layer's activations (2 nfilters L order fp32-sized values) and the weights re-split for the matrix cores
+ * (2 nfilters x (2 layers x 3 bf16 parts x order^2 + 2 bf16 parts x d x order)). */
+size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int d, int order);
 
 /* taps[f] (d, 2L) fp32, f < nfilters:  taps[f][c][l]      = k_fwd[c][l]       for l < L
  *                                      taps[f][c][L + l]  = k_rev[c][L-1-l]   (0 if not bidirectional)
@@ -79,12 +79,12 @@ int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int 
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The intermediate activations
  * go through a device array of M2_HYENA_FILTER_STATIC_SCRATCH_BYTES that is part of the library itself (every GPU
  * the library runs on holds one copy until the process ends); the call allocates and frees nothing.  Limit:
- * m2_hyena_filter_workspace_bytes(nfilters, L, order) must not exceed that size, i.e. nfilters * L <= 16384 (both
- * filters of a mixer up to L = 8192); beyond it the call fails with M2_ERR_UNSUPPORTED.  All calls on one GPU share
+ * m2_hyena_filter_workspace_bytes(nfilters, L, d, order) must not exceed that size, which at d = 768 means
+ * nfilters * L <= 16384 (both filters of a mixer up to L = 8192); beyond it the call fails with M2_ERR_UNSUPPORTED.  All calls on one GPU share
  * the array: two such calls whose kernels may overlap on the same GPU (different streams, or different host threads
  * on different streams) race; calls on one stream are ordered and safe.  The first call on a device looks up the
  * array's device address (hipGetSymbolAddress): make that call outside a stream capture. */
-#define M2_HYENA_FILTER_STATIC_SCRATCH_BYTES (17u << 20)
+#define M2_HYENA_FILTER_STATIC_SCRATCH_BYTES (18u << 20)
 int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order,
                                int emb_dim, float w_mod, float shift, float* taps, void* stream);
 

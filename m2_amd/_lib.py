@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libm2_amd.so")
 
 M2_DTYPE_F32 = 0
 M2_DTYPE_BF16 = 1
-M2_HYENA_FILTER_STATIC_SCRATCH_BYTES = 17 << 20
+M2_HYENA_FILTER_STATIC_SCRATCH_BYTES = 18 << 20
 
 
 class HyenaFilterParams(ctypes.Structure):
@@ -34,7 +34,7 @@ def _load() -> ctypes.CDLL:
     lib.m2_version.restype = c_int
     lib.m2_last_error.restype = c_char_p
     lib.m2_hyena_filter_workspace_bytes.restype = c_size_t
-    lib.m2_hyena_filter_workspace_bytes.argtypes = [c_int, c_int, c_int]
+    lib.m2_hyena_filter_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int]
     lib.m2_hyena_filter_fwd.restype = c_int
     lib.m2_hyena_filter_fwd.argtypes = [POINTER(HyenaFilterParams), c_int, c_int, c_int, c_int, c_int, c_float,
                                         c_float, c_void_p, c_void_p, c_void_p]

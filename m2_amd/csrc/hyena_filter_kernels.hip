@@ -79,8 +79,32 @@ __device__ __forceinline__ void split3(float x, float& hi, float& mid, float& lo
 // The 128 x 128 weights of the two inner layers, split into three bf16 parts and laid out as MFMA A operands, so
 // that hidden_kernel fetches them with coalesced 16-byte loads and no arithmetic:
 // wsplit[mlp][layer][part][wave w][K step ks][lane (i, h)] = 8 bf16 of row 32 w + i, K = 16 ks + 8 h .. + 7.
+// The d x 128 output projection likewise, in two parts (hi, lo), for project_kernel:
+// w3split[mlp][part][32-channel tile][K step ks][lane (i, h)] = 8 bf16 of row 32 tile + i, K = 16 ks + 8 h .. + 7.
 constexpr int kSplitPerLayer = 3 * kOrder * kOrder;      // bf16 elements per (mlp, layer)
-__global__ __launch_bounds__(256) void split_weights_kernel(FilterBatch fb, int nmlp, uint16_t* __restrict__ wsplit) {
+__global__ __launch_bounds__(256) void split_weights_kernel(FilterBatch fb, int nmlp, int d, uint16_t* __restrict__ wsplit,
+                                                            uint16_t* __restrict__ w3split) {
+  const int inner_blocks = nmlp * 2 * 4 * 8 * 64 / 256;
+  if ((int)blockIdx.x >= inner_blocks) {
+    const int id = ((int)blockIdx.x - inner_blocks) * 256 + threadIdx.x;      // (mlp, channel tile, ks, lane)
+    const int lane = id & 63, ks = (id >> 6) & 7, ct = (id >> 9) % (d / 32), m = (id >> 9) / (d / 32);
+    if (m >= nmlp) return;
+    const MlpPtrs& W = fb.f[m >> 1].mlp[m & 1];
+    if (W.w3 == nullptr) return;
+    const float* src = W.w3 + (long)(32 * ct + (lane & 31)) * kOrder + 16 * ks + 8 * (lane >> 5);
+    float h[8], l[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      h[j] = bf16_to_f32(f32_to_bf16(src[j]));
+      l[j] = src[j] - h[j];
+    }
+    u32x4* dst = reinterpret_cast<u32x4*>(w3split + (long)m * 2 * d * kOrder) + (ct * 8 + ks) * 64 + lane;
+    const u32x4 vh = {pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]), pack_bf16x2(h[4], h[5]), pack_bf16x2(h[6], h[7])};
+    const u32x4 vl = {pack_bf16x2(l[0], l[1]), pack_bf16x2(l[2], l[3]), pack_bf16x2(l[4], l[5]), pack_bf16x2(l[6], l[7])};
+    dst[0] = vh;
+    dst[d * kOrder / 8] = vl;
+    return;
+  }
   const int id = blockIdx.x * 256 + threadIdx.x;             // (mlp, layer, wave, ks, lane)
   const int lane = id & 63, ks = (id >> 6) & 7, w = (id >> 9) & 3, layer = (id >> 11) & 1, m = id >> 12;
   if (m >= nmlp) return;
@@ -265,6 +289,7 @@ constexpr int kPosPerWg = 256;      // at most; 32-position tiles past L are ski
 constexpr int kHRow = 2 * kOrder + 16;   // bytes per padded LDS row of one h3 part
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) void project_kernel(FilterBatch fb, int L, int d, float shift,
                                                       const uint16_t* __restrict__ h_hi, const uint16_t* __restrict__ h_lo,
+                                                      const uint16_t* __restrict__ w3split,
                                                       float* __restrict__ taps /* (nf, d, 2L) */) {
   __shared__ __attribute__((aligned(16))) unsigned char hbuf[2][2][32 * kHRow];     // [buffer][hi, lo][row]
   const int fi = blockIdx.z >> 1, dir = blockIdx.z & 1;
@@ -309,24 +334,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
   fetch(0, ic<0>{});
   if (ntiles > 1) fetch(1, ic<1>{});
 
-  // A operand: rows c0 + i32, K = 16 ks + 8 half + {0..7}, split hi / lo
+  // A operand: rows c0 + i32, K = 16 ks + 8 half + {0..7}, hi / lo parts as split_weights_kernel laid them out
   bf16x8 ahi[kOrder / 16], alo[kOrder / 16];
   float adelta[16];
   if (active) {
-    const float* wr = F.mlp[dir].w3 + (long)(c0 + i32) * kOrder + 8 * half;
+    const u32x4* wp = reinterpret_cast<const u32x4*>(w3split + (long)blockIdx.z * 2 * d * kOrder) + (c0 / 32) * 8 * 64 + lane;
 #pragma unroll
     for (int ks = 0; ks < kOrder / 16; ++ks) {
-      const float4 v0 = *reinterpret_cast<const float4*>(wr + 16 * ks);
-      const float4 v1 = *reinterpret_cast<const float4*>(wr + 16 * ks + 4);
-      const float x[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-      float h[8], l[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        h[j] = bf16_to_f32(f32_to_bf16(x[j]));
-        l[j] = x[j] - h[j];
-      }
-      ahi[ks] = as_bf16x8(pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3]), pack_bf16x2(h[4], h[5]), pack_bf16x2(h[6], h[7]));
-      alo[ks] = as_bf16x8(pack_bf16x2(l[0], l[1]), pack_bf16x2(l[2], l[3]), pack_bf16x2(l[4], l[5]), pack_bf16x2(l[6], l[7]));
+      ahi[ks] = __builtin_bit_cast(bf16x8, wp[ks * 64]);
+      alo[ks] = __builtin_bit_cast(bf16x8, wp[ks * 64 + d * kOrder / 8]);
     }
 #pragma unroll
     for (int v = 0; v < 16; ++v) adelta[v] = -fabsf(F.deltas[c0 + 8 * (v >> 2) + 4 * half + (v & 3)]) * 1.44269504088896341f;
@@ -378,10 +394,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
 
 using namespace m2;
 
-extern "C" size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int order) {
-  if (nfilters <= 0 || L <= 0 || order <= 0) return 0;
-  // h3 as bf16 hi / lo parts, then the inner-layer weights of the 2 nfilters MLPs as three bf16 parts each
-  return (size_t)2 * nfilters * L * order * sizeof(float) + (size_t)2 * nfilters * 2 * 3 * order * order * sizeof(uint16_t);
+extern "C" size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int d, int order) {
+  if (nfilters <= 0 || L <= 0 || d <= 0 || order <= 0) return 0;
+  // h3 as bf16 hi / lo parts; the inner-layer weights of the 2 nfilters MLPs as three bf16 parts each; their output
+  // projections as two
+  return (size_t)2 * nfilters * L * order * sizeof(float) + (size_t)2 * nfilters * 2 * 3 * order * order * sizeof(uint16_t) +
+         (size_t)2 * nfilters * 2 * d * order * sizeof(uint16_t);
 }
 
 // Shared by the two entry points: validation and the two launches, `workspace` holding the h3 hi / lo parts.
@@ -413,7 +431,9 @@ static int hyena_filter_launch(const char* who, const m2_hyena_filter_params* pa
   uint16_t* h_hi = reinterpret_cast<uint16_t*>(workspace);
   uint16_t* h_lo = h_hi + (size_t)2 * nfilters * L * order;
   uint16_t* wsplit = h_lo + (size_t)2 * nfilters * L * order;
-  hipLaunchKernelGGL(split_weights_kernel, dim3(2 * nfilters * 2 * 4 * 8 * 64 / 256), dim3(256), 0, s, fb, 2 * nfilters, wsplit);
+  uint16_t* w3split = wsplit + (size_t)2 * nfilters * 2 * 3 * order * order;
+  const int split_blocks = 2 * nfilters * 2 * 4 * 8 * 64 / 256 + 2 * nfilters * (d / 32) * 8 * 64 / 256;
+  hipLaunchKernelGGL(split_weights_kernel, dim3(split_blocks), dim3(256), 0, s, fb, 2 * nfilters, d, wsplit, w3split);
   int rc = check_launch("hyena split_weights_kernel");
   if (rc) return rc;
   // positions per workgroup: longer runs amortise the weight fetch (96 KB per workgroup and layer), short sequences
@@ -425,7 +445,7 @@ static int hyena_filter_launch(const char* who, const m2_hyena_filter_params* pa
   rc = check_launch("hyena hidden_kernel");
   if (rc) return rc;
   hipLaunchKernelGGL(project_kernel, dim3((L + kPosPerWg - 1) / kPosPerWg, (d + 127) / 128, 2 * nfilters), dim3(256), 0, s, fb, L, d, shift,
-                     h_hi, h_lo, taps);
+                     h_hi, h_lo, w3split, taps);
   return check_launch("hyena project_kernel");
 }
 
@@ -477,13 +497,12 @@ extern "C" int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, 
   if (!params || !taps) return set_error(M2_ERR_ARG, "m2_hyena_filter_fwd_static: null pointer");
   if (nfilters < 1 || L <= 0 || order <= 0)
     return set_error(M2_ERR_ARG, "m2_hyena_filter_fwd_static: sizes must be positive (nfilters=%d L=%d order=%d)", nfilters, L, order);
-  const size_t need = m2_hyena_filter_workspace_bytes(nfilters, L, order);
+  const size_t need = m2_hyena_filter_workspace_bytes(nfilters, L, d, order);
   if (need > (size_t)M2_HYENA_FILTER_STATIC_SCRATCH_BYTES)
     return set_error(M2_ERR_UNSUPPORTED,
                      "m2_hyena_filter_fwd_static: nfilters=%d, L=%d needs %zu bytes of scratch, the static array holds %zu "
-                     "(nfilters * L <= %zu); use m2_hyena_filter_fwd with a caller workspace",
-                     nfilters, L, need, (size_t)M2_HYENA_FILTER_STATIC_SCRATCH_BYTES,
-                     (size_t)M2_HYENA_FILTER_STATIC_SCRATCH_BYTES / (2 * kOrder * sizeof(float)));
+                     "(m2_hyena_filter_workspace_bytes); use m2_hyena_filter_fwd with a caller workspace",
+                     nfilters, L, need, (size_t)M2_HYENA_FILTER_STATIC_SCRATCH_BYTES);
   void* ptr = nullptr;
   int rc = static_scratch_for_current_device(&ptr);
   if (rc) return rc;

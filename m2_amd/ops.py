@@ -98,7 +98,7 @@ def hyena_filter_taps(filters: Sequence[dict], L: int, d: int, order: int, emb_d
         check(lib.m2_hyena_filter_fwd_static(arr, nf, L, d, order, emb_dim, float(w_mod), float(shift), _ptr(taps),
                                              _stream()))
         return taps
-    ws_bytes = lib.m2_hyena_filter_workspace_bytes(nf, L, order)
+    ws_bytes = lib.m2_hyena_filter_workspace_bytes(nf, L, d, order)
     workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
     check(lib.m2_hyena_filter_fwd(arr, nf, L, d, order, emb_dim, float(w_mod), float(shift), _ptr(workspace),
                                   _ptr(taps), _stream()))

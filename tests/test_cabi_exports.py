@@ -42,7 +42,8 @@ def test_size_queries_and_argument_checks_without_gpu():
     assert lib.m2_fftconv_supported_seqlen(64) == 0
     assert lib.m2_fftconv_supported_seqlen(100) == 0
     assert lib.m2_filter_spectrum_bytes(768, 8192) == 768 * 8192 * 16
-    assert lib.m2_hyena_filter_workspace_bytes(2, 8192, 128) == 2 * 2 * 8192 * 128 * 4 + 2 * 2 * 2 * 3 * 128 * 128 * 2
+    assert lib.m2_hyena_filter_workspace_bytes(2, 8192, 768, 128) == (2 * 2 * 8192 * 128 * 4 + 2 * 2 * 2 * 3 * 128 * 128 * 2
+                                                                      + 2 * 2 * 2 * 768 * 128 * 2)
     # null pointers and unsupported sizes are refused before anything is launched
     assert lib.m2_mixer_core_fwd(None, None, None, None, None, None, None, 1, 128, 64, 0, None) == -1
     assert b"null" in lib.m2_last_error()

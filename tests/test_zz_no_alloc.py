@@ -26,7 +26,7 @@ def test_static_scratch_entry_point_matches_workspace_entry_point(gpu):
     cfg.hidden_size = d
     filters, _ = _filters(cfg, 3, gpu)
     for L in (8192, 1024):                       # the second call is shorter: stale scratch beyond it must not matter
-        assert lib.m2_hyena_filter_workspace_bytes(2, L, 128) <= M2_HYENA_FILTER_STATIC_SCRATCH_BYTES
+        assert lib.m2_hyena_filter_workspace_bytes(2, L, d, 128) <= M2_HYENA_FILTER_STATIC_SCRATCH_BYTES
         want = ops.hyena_filter_taps(filters, L, d, 128, 5)
         out = torch.full((2, d, 2 * L), float("nan"), device=gpu)
         free_before = torch.cuda.mem_get_info()[0]
