@@ -199,6 +199,10 @@ int m2_mlp_fused_fwd(const void* x, const void* w_packed, const float* bias, con
  * layout m2_mixer_core_fwd reads its `u` in).  Needs d % 64 == 0, d <= 2048. */
 int m2_layernorm_fwd(const float* x, const float* gamma, const float* beta, float eps, float* out_f32, void* out_bf16,
                      float* out_channel_major, int M, int d, void* stream);
+/* The same for x (M, d) stored as bf16: what the reference's LayerNorm receives under CUDA autocast, where the sum
+ * wo(...) + residual is a bf16 tensor (bert/src/bert_layers.py:504-506); statistics and outputs in fp32 as above. */
+int m2_layernorm_bf16_fwd(const void* x, const float* gamma, const float* beta, float eps, float* out_f32,
+                          void* out_bf16, float* out_channel_major, int M, int d, void* stream);
 
 /* out = LayerNorm(blockdiag_multiply(x, w) + bias + residual) in one kernel: m2_blockdiag_linear_fwd followed by
  * m2_layernorm_fwd without the fp32 intermediate (bert/src/bert_layers.py:504-506: wo, dropout, residual,

@@ -484,8 +484,9 @@ __device__ __forceinline__ long long clamp_index(long long i, int rows, bool& ba
   }
   return i;
 }
-template <int PER, bool EMBED>
-__global__ __launch_bounds__(512) void layernorm_kernel(const float* __restrict__ x, EmbedSource src,
+// IN: float, or uint16_t for rows stored as bf16 (the sum the reference's autocast path feeds its LayerNorm).
+template <int PER, bool EMBED, typename IN = float>
+__global__ __launch_bounds__(512) void layernorm_kernel(const IN* __restrict__ x, EmbedSource src,
                                                         const float* __restrict__ gamma,
                                                         const float* __restrict__ beta, float eps,
                                                         float* __restrict__ out_f32,       // (M, d) or null
@@ -509,8 +510,11 @@ __global__ __launch_bounds__(512) void layernorm_kernel(const float* __restrict_
     int m = m0 + wave * RW + rr;
     m = m < M ? m : M - 1;
     if constexpr (!EMBED) {
-      const float* xr = x + (long)m * d;
-      static_for<0, PER>([&](auto ii) { v[rr][decltype(ii)::value] = xr[lane + 64 * decltype(ii)::value]; });
+      const IN* xr = x + (long)m * d;
+      static_for<0, PER>([&](auto ii) {
+        if constexpr (sizeof(IN) == 2) v[rr][decltype(ii)::value] = bf16_to_f32(xr[lane + 64 * decltype(ii)::value]);
+        else v[rr][decltype(ii)::value] = xr[lane + 64 * decltype(ii)::value];
+      });
     } else {
       bool bad = false;
       const float* wr = src.word + clamp_index(src.ids[m], src.vocab, bad) * d;
@@ -1012,8 +1016,8 @@ extern "C" int m2_blockdiag_linear_f32_fwd(const float* x, const float* w, const
   return check_launch("blockdiag_f32");
 }
 
-template <bool EMBED>
-static int launch_layernorm(const float* x, const EmbedSource& src, const float* gamma, const float* beta, float eps,
+template <bool EMBED, typename IN = float>
+static int launch_layernorm(const IN* x, const EmbedSource& src, const float* gamma, const float* beta, float eps,
                             float* out_f32, void* out_bf16, float* out_channel_major, int M, int d, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   uint16_t* o16 = (uint16_t*)out_bf16;
@@ -1021,7 +1025,7 @@ static int launch_layernorm(const float* x, const EmbedSource& src, const float*
 #define LN_CASE(P)                                                                                                      \
   case P: {                                                                                                             \
     const size_t lds = out_channel_major ? LnShape<P>::LDS_BYTES : 0;                                                   \
-    auto kern = layernorm_kernel<P, EMBED>;                                                                             \
+    auto kern = layernorm_kernel<P, EMBED, IN>;                                                                           \
     if (lds > 64 * 1024) {                                                                                              \
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
       if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(layernorm): %s", hipGetErrorString(e)); \
@@ -1047,6 +1051,15 @@ extern "C" int m2_layernorm_fwd(const float* x, const float* gamma, const float*
   return launch_layernorm<false>(x, EmbedSource{}, gamma, beta, eps, out_f32, out_bf16, out_channel_major, M, d, stream);
 }
 
+extern "C" int m2_layernorm_bf16_fwd(const void* x, const float* gamma, const float* beta, float eps, float* out_f32,
+                                     void* out_bf16, float* out_channel_major, int M, int d, void* stream) {
+  if (!x || !gamma || !beta) return set_error(M2_ERR_ARG, "m2_layernorm_bf16_fwd: null pointer");
+  if (M <= 0 || d <= 0 || d % 64 != 0 || d > 2048)
+    return set_error(M2_ERR_UNSUPPORTED, "m2_layernorm_bf16_fwd: need M > 0 and d a multiple of 64 up to 2048 (M=%d d=%d)", M, d);
+  return launch_layernorm<false, uint16_t>((const uint16_t*)x, EmbedSource{}, gamma, beta, eps, out_f32, out_bf16,
+                                           out_channel_major, M, d, stream);
+}
+
 extern "C" int m2_embed_layernorm_fwd(const long long* input_ids, const long long* token_type_ids,
                                       const long long* position_ids, const float* word_emb, const float* type_emb,
                                       const float* pos_emb, int vocab_size, int type_vocab_size, int max_positions,
@@ -1065,5 +1078,5 @@ extern "C" int m2_embed_layernorm_fwd(const long long* input_ids, const long lon
     return set_error(M2_ERR_ARG, "m2_embed_layernorm_fwd: sequence length %d exceeds the position table (%d rows)", L, max_positions);
   const EmbedSource src{input_ids, token_type_ids, position_ids, word_emb, type_emb, pos_emb, L,
                         vocab_size, type_vocab_size, max_positions, bad_index};
-  return launch_layernorm<true>(nullptr, src, gamma, beta, eps, out_f32, out_bf16, out_channel_major, B * L, d, stream);
+  return launch_layernorm<true>((const float*)nullptr, src, gamma, beta, eps, out_f32, out_bf16, out_channel_major, B * L, d, stream);
 }

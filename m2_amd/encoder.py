@@ -138,20 +138,26 @@ class BertGatedLinearUnitMLP(nn.Module):
     # I = 3072) that is rebuilt when the weights change.
     fuse_mlp = True
     _packed = None
+    # True: the sum wo(...) + bias + residual goes to the LayerNorm as bf16 instead of fp32 -- the rounding the
+    # reference's autocast path applies at this point (its wo output, residual and their sum are bf16 tensors) --
+    # which halves the bytes written by the MLP kernel and read by the LayerNorm: -1.9 % per forward at L = 8192,
+    # B = 4; per-layer deviation from the fp32 oracle 0.89 % instead of 0.78 % (max), end to end unchanged.
+    bf16_presum = True
 
     def presum(self, a16: torch.Tensor) -> torch.Tensor:
-        """a16 (M, d) bf16 -> wo(glu(a16)) + bias + a16, (M, d) fp32 (the LayerNorm input)."""
+        """a16 (M, d) bf16 -> wo(glu(a16)) + bias + a16, (M, d) fp32 (the LayerNorm input; bf16 with `bf16_presum`)."""
+        sum_dtype = torch.bfloat16 if self.bf16_presum else torch.float32
         if self.fuse_mlp and ops.mlp_fused_supported(a16.shape[1], self.config.intermediate_size,
                                                      self.config.monarch_mlp_nblocks):
             wg, wo = self.gated_layers.weight_bf16(), self.wo.weight_bf16()
             # the packed copy the kernel streams: rebuilt whenever one of the bf16 copies has been rebuilt
             if self._packed is None or self._packed[0] is not wg or self._packed[1] is not wo:
                 self._packed = (wg, wo, ops.mlp_fused_pack(wg, wo))
-            return ops.mlp_fused(a16, wg, wo, self.wo.bias.detach().float().contiguous(), a16, out_dtype=torch.float32,
+            return ops.mlp_fused(a16, wg, wo, self.wo.bias.detach().float().contiguous(), a16, out_dtype=sum_dtype,
                                  packed=self._packed[2])
         g = ops.blockdiag_glu(a16, self.gated_layers.weight_bf16())
         return ops.blockdiag_linear(g, self.wo.weight_bf16(), self.wo.bias.detach().float().contiguous(), a16,
-                                    out_dtype=torch.float32)
+                                    out_dtype=sum_dtype)
 
     def ln_params(self):
         return self.layernorm.weight.detach().float(), self.layernorm.bias.detach().float(), self.layernorm.eps

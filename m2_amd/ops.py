@@ -274,16 +274,19 @@ def mlp_fused(x: Tensor, w_gated: Tensor, w_out: Tensor, bias: Optional[Tensor] 
 
 def layernorm(x: Tensor, gamma: Tensor, beta: Tensor, eps: float, want_f32: bool = True, want_bf16: bool = False,
               want_channel_major: bool = False):
-    """LayerNorm over the last dim of x (M, d) fp32 -> (f32 (M,d) | None, bf16 (M,d) | None, f32 (d,M) | None)."""
+    """LayerNorm over the last dim of x (M, d) fp32 or bf16 -> (f32 (M,d) | None, bf16 (M,d) | None, f32 (d,M) | None)."""
     M, d = x.shape
-    _require(x, "x", torch.float32)
+    if x.dtype != torch.bfloat16:
+        _require(x, "x", torch.float32)
+    else:
+        _require(x, "x", torch.bfloat16)
     _require(gamma, "gamma", torch.float32, (d,))
     _require(beta, "beta", torch.float32, (d,))
     o32 = torch.empty(M, d, dtype=torch.float32, device=x.device) if want_f32 else None
     o16 = torch.empty(M, d, dtype=torch.bfloat16, device=x.device) if want_bf16 else None
     ot = torch.empty(d, M, dtype=torch.float32, device=x.device) if want_channel_major else None
-    check(lib.m2_layernorm_fwd(_ptr(x), _ptr(gamma), _ptr(beta), float(eps), _ptr(o32), _ptr(o16), _ptr(ot), M, d,
-                               _stream()))
+    fn = lib.m2_layernorm_bf16_fwd if x.dtype == torch.bfloat16 else lib.m2_layernorm_fwd
+    check(fn(_ptr(x), _ptr(gamma), _ptr(beta), float(eps), _ptr(o32), _ptr(o16), _ptr(ot), M, d, _stream()))
     return o32, o16, ot
 
 

@@ -156,6 +156,14 @@ def test_layernorm_three_outputs(gpu, M, d):
     assert rel_err(o32, ref)[0] < 1e-5
     assert rel_err(ot.T, ref)[0] < 1e-5
     assert rel_err(o16.float(), ref)[0] < 6e-3
+    # rows stored as bf16 (what the reference's LayerNorm receives under autocast): the same statistics in fp32 on
+    # the rounded values
+    x16 = x.bfloat16()
+    p32, p16, pt = ops.layernorm(x16.to(gpu), gamma.to(gpu), beta.to(gpu), 1e-12, True, True, True)
+    ref16 = torch.nn.functional.layer_norm(x16.double(), (d,), gamma.double(), beta.double(), 1e-12)
+    assert rel_err(p32, ref16)[0] < 1e-5
+    assert rel_err(pt.T, ref16)[0] < 1e-5
+    assert rel_err(p16.float(), ref16)[0] < 6e-3
 
 
 def test_config1_mixer_fp32(gpu):
