@@ -48,7 +48,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM-side bytes per mixer-core launch at the default workload, from the two rocprofv3 --pmc runs
 # (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000 against a plain 256 MiB copy); summary in
 # profiles/encoder_fwd_L8192_B4_hbm_traffic.md.  Only valid for --config c3.
-MIXER_CORE_TRAFFIC_BYTES_C3 = int((189581 * 2.0 + 55574 * 1.0) * 1024)
+MIXER_CORE_TRAFFIC_BYTES_C3 = int((190182 * 2.0 + 55629 * 1.0) * 1024)
 
 
 REFERENCE_GRID = {"l512": (512, 32), "l1024": (1024, 32), "l2048": (2048, 16), "l4096": (4096, 8)}
