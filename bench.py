@@ -176,7 +176,34 @@ def probe_matrix_pipe(iters: int = 4000):
             rows.append({"lds_reads_per_mfma": reads, "valu_per_mfma": valu, "waves_per_simd": wps, "ms": ms,
                          "tflops": tflops, "frac_of_published_peak": tflops / MFMA_BF16_PEAK_TFLOPS})
     return {"probe": "v_mfma_f32_32x32x16_bf16 loop on all compute units", "published_peak_tflops": MFMA_BF16_PEAK_TFLOPS,
-            "rows": rows, "dft16_pass": probe_dft16_pass()}
+            "rows": rows, "dft16_pass": probe_dft16_pass(), "l2_stream": probe_l2_stream()}
+
+
+def probe_l2_stream(iters: int = 2000):
+    """What one compute unit pulls out of L2 into LDS when all of them do (m2_probe_l2_stream_fwd)."""
+    import ctypes
+    from m2_amd._lib import check, lib
+    region = torch.ones(1 << 20, device="cuda:0", dtype=torch.float32)      # 4 MiB
+    sink = torch.zeros(512, device="cuda:0")
+    out = []
+    for mode, name in ((0, "direct-to-LDS loads, sixteen 64-byte row pieces per instruction"),
+                       (1, "direct-to-LDS loads, 1 KB contiguous per instruction"),
+                       (2, "plain 16-byte loads, software-pipelined, then LDS writes")):
+        wgs = ctypes.c_int(0)
+        call = lambda it: check(lib.m2_probe_l2_stream_fwd(mode, it, ctypes.c_void_p(region.data_ptr()), 1 << 20,
+                                                           ctypes.c_void_p(sink.data_ptr()), ctypes.byref(wgs),
+                                                           torch.cuda.current_stream().cuda_stream))
+        call(10)
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        call(iters)
+        e.record()
+        torch.cuda.synchronize()
+        us_per_iter = s.elapsed_time(e) * 1e3 / iters
+        out.append({"mode": name, "us_per_40KB": us_per_iter, "GBps_per_compute_unit": 40960 / us_per_iter / 1e3,
+                    "TBps_all": wgs.value * 40960 / us_per_iter / 1e6, "workgroups": wgs.value})
+    return out
 
 
 def probe_dft16_pass(nrows: int = 1024, iters: int = 200):

@@ -169,6 +169,65 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   for (int i = t; i < P::L; i += 256) g[i] = row[sphys(i)];
 }
 
+// ---------------------------------------------------------------------------------------------
+// L2 -> LDS stream: what one compute unit can pull out of L2 when all of them do.  Every workgroup (512 threads, one
+// per compute unit) copies the same `region` (so everything is an L2 hit after the first pass) into LDS, 40 KB per
+// iteration, a barrier per iteration, in one of three ways:
+//   mode 0  direct loads (global_load_lds_dwordx4), an instruction gathering sixteen 64-byte row pieces (row stride
+//           384 bytes: an MFMA operand block taken straight from a row-major bf16 matrix with 192 columns)
+//   mode 1  direct loads, an instruction copying 1 KB of contiguous memory
+//   mode 2  plain 16-byte loads into registers, software-pipelined one iteration ahead, then LDS writes
+// ---------------------------------------------------------------------------------------------
+template <int MODE>
+__global__ __launch_bounds__(512) void probe_l2_stream_kernel(const unsigned char* __restrict__ src, long region, int iters,
+                                                              float* __restrict__ sink) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char stage[];      // 4 stages x 40 KB
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const unsigned lds0 = (unsigned)(uintptr_t)stage;
+  const unsigned voff = MODE == 0 ? (lane & 15) * 384 + (lane >> 4) * 16 : lane * 16;
+  const long span = region - 16 * 384 - 1024;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  if constexpr (MODE < 2) {
+    long off = 0;
+    for (int it = 0; it < iters; ++it) {
+      for (int j = 0; j < 5; ++j) {
+        const int blk = wave * 5 + j;
+        long o = MODE == 0 ? (blk % 6) * 64 + (long)((blk / 6) * 16) * 384 + off : off + (long)blk * 1024;
+        o %= span;
+        const unsigned dst = lds0 + ((it & 3) * 40 + blk) * 1024;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff), "s"(src + o) : "memory");
+      }
+      off += MODE == 0 ? 384 * 32 : 40 * 1024;
+      __builtin_amdgcn_s_waitcnt(0x0F70 | 5);      // all but the newest batch have landed
+      __syncthreads();
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+  } else {
+    u32x4 ra[5], rb[5];
+    auto ld = [&](u32x4* r, int it) __attribute__((always_inline)) {
+#pragma unroll
+      for (int j = 0; j < 5; ++j) r[j] = *reinterpret_cast<const u32x4*>(src + ((long)it * 40 * 1024 + (long)(wave * 5 + j) * 1024) % span + voff);
+    };
+    auto st = [&](const u32x4* r, int it) __attribute__((always_inline)) {
+#pragma unroll
+      for (int j = 0; j < 5; ++j) *reinterpret_cast<u32x4*>(stage + ((it & 3) * 40 + wave * 5 + j) * 1024 + lane * 16) = r[j];
+    };
+    ld(ra, 0);
+    for (int it = 0; it < iters; it += 2) {
+      ld(rb, it + 1);
+      st(ra, it);
+      __syncthreads();
+      ld(ra, it + 2);
+      st(rb, it + 1);
+      __syncthreads();
+    }
+    if (ra[0].x == 0x12345678u) sink[tid] = 2.f;
+  }
+  __syncthreads();
+  if (*reinterpret_cast<const uint32_t*>(stage + 16 * tid) == 0x12345678u) sink[tid] = 1.f;
+}
+
 }  // namespace m2
 
 using namespace m2;
@@ -197,4 +256,19 @@ extern "C" int m2_probe_dft16_pass_fwd(int use_mfma, int iters, int nrows, float
   if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(probe_dft16): %s", hipGetErrorString(e));
   hipLaunchKernelGGL(kern, dim3(nrows), dim3(256), lds, (hipStream_t)stream, reinterpret_cast<float2*>(rows), iters);
   return check_launch("probe_dft16");
+}
+
+extern "C" int m2_probe_l2_stream_fwd(int mode, int iters, const void* region, long region_bytes, float* sink, int* workgroups,
+                                      void* stream) {
+  if (!region || !sink || iters <= 0) return set_error(M2_ERR_ARG, "m2_probe_l2_stream_fwd: null pointer or non-positive iters");
+  if (region_bytes < (1 << 20)) return set_error(M2_ERR_ARG, "m2_probe_l2_stream_fwd: region of %ld bytes, need at least 1 MiB", region_bytes);
+  if (mode < 0 || mode > 2) return set_error(M2_ERR_UNSUPPORTED, "m2_probe_l2_stream_fwd: mode must be 0, 1 or 2");
+  const int lds = 160 * 1024;
+  auto kern = mode == 0 ? probe_l2_stream_kernel<0> : mode == 1 ? probe_l2_stream_kernel<1> : probe_l2_stream_kernel<2>;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(probe_l2_stream): %s", hipGetErrorString(e));
+  if (workgroups) *workgroups = num_cus();
+  hipLaunchKernelGGL(kern, dim3(num_cus()), dim3(512), lds, (hipStream_t)stream, (const unsigned char*)region, region_bytes,
+                     iters & ~1, sink);
+  return check_launch("probe_l2_stream");
 }
