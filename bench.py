@@ -188,7 +188,8 @@ def probe_l2_stream(iters: int = 2000):
     out = []
     for mode, name in ((0, "direct-to-LDS loads, sixteen 64-byte row pieces per instruction"),
                        (1, "direct-to-LDS loads, 1 KB contiguous per instruction"),
-                       (2, "plain 16-byte loads, software-pipelined, then LDS writes")):
+                       (2, "plain 16-byte loads, software-pipelined, then LDS writes"),
+                       (3, "direct-to-LDS loads, eight whole 128-byte lines per instruction")):
         wgs = ctypes.c_int(0)
         call = lambda it: check(lib.m2_probe_l2_stream_fwd(mode, it, ctypes.c_void_p(region.data_ptr()), 1 << 20,
                                                            ctypes.c_void_p(sink.data_ptr()), ctypes.byref(wgs),

@@ -254,8 +254,8 @@ int m2_probe_dft16_pass_fwd(int use_mfma, int iters, int nrows, float* rows, voi
 /* Measurement probe: the L2 -> LDS stream one compute unit sustains when all do.  One 512-thread workgroup per
  * compute unit copies the same `region` (>= 1 MiB of device memory, L2-resident after the first pass) into LDS,
  * 40 KB per iteration with a barrier, by direct-to-LDS loads that gather sixteen 64-byte row pieces per instruction
- * (mode 0), direct-to-LDS loads of 1 KB contiguous per instruction (mode 1), or software-pipelined plain loads
- * followed by LDS writes (mode 2).  `sink`: 512 floats; *workgroups receives the number of workgroups launched.
+ * (mode 0), direct-to-LDS loads of 1 KB contiguous per instruction (mode 1), software-pipelined plain loads
+ * followed by LDS writes (mode 2), or direct-to-LDS loads that gather eight whole 128-byte lines (mode 3).  `sink`: 512 floats; *workgroups receives the number of workgroups launched.
  * Bytes moved = workgroups * iters * 40960. */
 int m2_probe_l2_stream_fwd(int mode, int iters, const void* region, long region_bytes, float* sink, int* workgroups,
                            void* stream);

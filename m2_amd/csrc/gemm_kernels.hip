@@ -9,8 +9,10 @@
 // Workgroup = 8 waves (two per SIMD) on a 256 (q) x 256 (p) tile, wave (wq, wp) = 64 x 128: 2 x 4 MFMA tiles of
 // v_mfma_f32_32x32x16_bf16, 128 accumulators per lane.  K advances in chunks of 64 through two LDS stages of 64 KB
 // that are written by direct global -> LDS loads (global_load_lds_dwordx4: no staging registers, no LDS write
-// instructions); a stage is laid out [32-row block][K step][lane], so every MFMA operand is one conflict-free
-// 16-byte LDS read.  Operand registers are double-buffered per K step: the reads of step s + 1 are issued before
+// instructions).  A load instruction fetches eight rows x 128 bytes, i.e. eight whole cache lines (the L2 delivers
+// whole-line gathers at twice the rate of 32- or 64-byte row pieces: measured); the 16-byte pieces of such a block are
+// placed [K step][half][row], with the two halves swapped in every other block, so that an MFMA operand -- 32 rows x
+// one K step, four blocks -- is one 16-byte LDS read per lane that touches every bank once per 16 lanes.  Operand registers are double-buffered per K step: the reads of step s + 1 are issued before
 // the eight MFMAs of step s (6 reads per 8 MFMAs).  The finished tile goes through LDS so that every global store
 // is a full row segment.
 #include <hip/hip_runtime.h>
@@ -27,9 +29,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kGT = 256;                    // tile edge (both ways)
 constexpr int kGK = 64;                     // K per chunk
-constexpr int kGBlk = 1024;                 // one operand block: 64 lanes x 16 bytes = 32 rows x 16 K
-constexpr int kGSide = (kGT / 32) * (kGK / 16) * kGBlk;      // P (or Q) part of a stage: 32 KB
+constexpr int kGBlk = 1024;                 // one load instruction: 64 lanes x 16 bytes = 8 rows x 64 K
+constexpr int kGSide = (kGT / 8) * kGBlk;   // P (or Q) part of a stage: 32 blocks = 32 KB
 constexpr int kGStage = 2 * kGSide;         // 64 KB
+constexpr int kGStages = 2;
 constexpr int kGOutRow = 2 * kGT + 16;      // bytes per padded row of the bf16 output tile in LDS
 constexpr int kGLds = kGT * kGOutRow;       // 135168 bytes >= 2 stages
 
@@ -70,26 +73,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int p0 = tp * kGT, q0 = tq * kGT;
   const int nchunks = g.K / kGK;
 
-  // ---- staging: a stage holds 32 P blocks then 32 Q blocks, block (rb, s) = rows [32 rb, +32), K step s of the
-  // chunk; wave w loads the blocks w, w + 8, ... of each side (4 + 4 per chunk).  Rows past the end are clamped.
+  // ---- staging: a stage holds 32 P blocks then 32 Q blocks, block b = rows [8 b, + 8) x the 64 K of the chunk; wave
+  // w loads the blocks w, w + 8, ... of each side (4 + 4 per chunk).  Lane l of a block = (K step l / 16, slot
+  // (l / 8) % 2, row l % 8); the slot holds K half (slot ^ b % 2), and b % 2 = w % 2 for all blocks of a wave.  Rows past
+  // the end are clamped.
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
   unsigned voff_p[4], voff_q[4];
   static_for<0, 4>([&](auto jj) {
     constexpr int j = decltype(jj)::value;
-    const int b = wave + 8 * j, rb = b >> 2, s = b & 3;
-    int rp = p0 + 32 * rb + i32, rq = q0 + 32 * rb + i32;
+    const int b = wave + 8 * j;
+    const int ks = lane >> 4, khalf = ((lane >> 3) & 1) ^ (wave & 1), r = lane & 7;
+    int rp = p0 + 8 * b + r, rq = q0 + 8 * b + r;
     rp = rp < g.np ? rp : g.np - 1;
     rq = rq < g.nq ? rq : g.nq - 1;
-    voff_p[j] = (unsigned)(((long)rp * g.ldp + 16 * s + 8 * half) * 2);
-    voff_q[j] = (unsigned)(((long)rq * g.ldq + 16 * s + 8 * half) * 2);
+    voff_p[j] = (unsigned)(((long)rp * g.ldp + 16 * ks + 8 * khalf) * 2);
+    voff_q[j] = (unsigned)(((long)rq * g.ldq + 16 * ks + 8 * khalf) * 2);
   });
-  auto dma = [&](int c) __attribute__((always_inline)) {
-    const unsigned st = __builtin_amdgcn_readfirstlane(lds0 + (c & 1) * kGStage + wave * kGBlk);
-    const uint16_t* bp = g.P + (long)c * kGK;
-    const uint16_t* bq = g.Q + (long)c * kGK;
-    static_for<0, 4>([&](auto jj) { gemm_load_to_lds(st + 8 * kGBlk * decltype(jj)::value, voff_p[decltype(jj)::value], bp); });
-    static_for<0, 4>([&](auto jj) { gemm_load_to_lds(st + kGSide + 8 * kGBlk * decltype(jj)::value, voff_q[decltype(jj)::value], bq); });
+  // loads j of chunk c: one P block and one Q block
+  auto dma_pair = [&](int c, auto jj) __attribute__((always_inline)) {
+    constexpr int j = decltype(jj)::value;
+    const unsigned st = __builtin_amdgcn_readfirstlane(lds0 + (c % kGStages) * kGStage + wave * kGBlk);
+    gemm_load_to_lds(st + 8 * kGBlk * j, voff_p[j], g.P + (long)c * kGK);
+    gemm_load_to_lds(st + kGSide + 8 * kGBlk * j, voff_q[j], g.Q + (long)c * kGK);
   };
+  auto dma = [&](int c) __attribute__((always_inline)) { static_for<0, 4>([&](auto jj) { dma_pair(c, jj); }); };
 
   floatx16 acc[2][4];      // [q tile][p tile]
   static_for<0, 8>([&](auto tt) {
@@ -100,7 +107,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   u32x4 opa[2][4], opb[2][2];
   auto read_ops = [&](int st, auto ss, auto bb) __attribute__((always_inline)) {
     constexpr int s = decltype(ss)::value, bf = decltype(bb)::value;
-    const unsigned char* base = smem + st * kGStage + 16 * lane + s * kGBlk;
+    // lane (i32, half) of a 32-row tile: block i32 / 8 of the tile's four, slot half ^ (block % 2), row i32 % 8
+    const unsigned char* base = smem + st * kGStage + (i32 >> 3) * kGBlk + (((half ^ ((i32 >> 3) & 1)) * 8 + (i32 & 7)) * 16) + s * 256;
     static_for<0, 4>([&](auto pp) {
       constexpr int pi = decltype(pp)::value;
       opa[bf][pi] = *reinterpret_cast<const u32x4*>(base + (4 * wp + pi) * 4 * kGBlk);
@@ -126,23 +134,29 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   for (int c = 0; c < nchunks; ++c) {
     __builtin_amdgcn_s_waitcnt(kGWaitVm0);      // this wave's pieces of chunk c have landed
     __syncthreads();                            // ... everybody's; and everybody is done reading chunk c - 1
-    if (c + 1 < nchunks) dma(c + 1);
     const int st = c & 1;
-    // the reads of K step s + 1 are issued before the MFMAs of step s (scheduling barriers pin that order)
+    const bool more = c + 1 < nchunks;
+    // The reads of K step s + 1 are issued before the MFMAs of step s (scheduling barriers pin that order), and the
+    // eight loads of the next chunk go out two at a time between the MFMA groups: issued together they fill the
+    // memory pipeline's queue and every wave stalls behind its own loads.
     read_ops(st, ic<0>{}, ic<0>{});
     __builtin_amdgcn_sched_barrier(0);
     read_ops(st, ic<1>{}, ic<1>{});
     __builtin_amdgcn_sched_barrier(0);
+    if (more) dma_pair(c + 1, ic<0>{});
     mfmas(ic<0>{});
     __builtin_amdgcn_sched_barrier(0);
     read_ops(st, ic<2>{}, ic<0>{});
     __builtin_amdgcn_sched_barrier(0);
+    if (more) dma_pair(c + 1, ic<1>{});
     mfmas(ic<1>{});
     __builtin_amdgcn_sched_barrier(0);
     read_ops(st, ic<3>{}, ic<1>{});
     __builtin_amdgcn_sched_barrier(0);
+    if (more) dma_pair(c + 1, ic<2>{});
     mfmas(ic<0>{});
     __builtin_amdgcn_sched_barrier(0);
+    if (more) dma_pair(c + 1, ic<3>{});
     mfmas(ic<1>{});
     __builtin_amdgcn_sched_barrier(0);
   }

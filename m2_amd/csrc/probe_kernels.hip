@@ -177,6 +177,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 //           384 bytes: an MFMA operand block taken straight from a row-major bf16 matrix with 192 columns)
 //   mode 1  direct loads, an instruction copying 1 KB of contiguous memory
 //   mode 2  plain 16-byte loads into registers, software-pipelined one iteration ahead, then LDS writes
+//   mode 3  direct loads, an instruction gathering eight whole 128-byte lines (row stride 1536 bytes: a 64-wide K
+//           chunk of eight rows of a row-major bf16 matrix with 768 columns)
 // ---------------------------------------------------------------------------------------------
 template <int MODE>
 __global__ __launch_bounds__(512) void probe_l2_stream_kernel(const unsigned char* __restrict__ src, long region, int iters,
@@ -185,20 +187,21 @@ __global__ __launch_bounds__(512) void probe_l2_stream_kernel(const unsigned cha
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const unsigned lds0 = (unsigned)(uintptr_t)stage;
-  const unsigned voff = MODE == 0 ? (lane & 15) * 384 + (lane >> 4) * 16 : lane * 16;
-  const long span = region - 16 * 384 - 1024;
+  const unsigned voff = MODE == 0 ? (lane & 15) * 384 + (lane >> 4) * 16 : MODE == 3 ? (lane >> 3) * 1536 + (lane & 7) * 16 : lane * 16;
+  const long span = region - 16 * 1536 - 1024;
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-  if constexpr (MODE < 2) {
+  if constexpr (MODE != 2) {
     long off = 0;
     for (int it = 0; it < iters; ++it) {
       for (int j = 0; j < 5; ++j) {
         const int blk = wave * 5 + j;
-        long o = MODE == 0 ? (blk % 6) * 64 + (long)((blk / 6) * 16) * 384 + off : off + (long)blk * 1024;
+        long o = MODE == 0 ? (blk % 6) * 64 + (long)((blk / 6) * 16) * 384 + off
+               : MODE == 3 ? (blk % 12) * 128 + (long)((blk / 12) * 8) * 1536 + off : off + (long)blk * 1024;
         o %= span;
         const unsigned dst = lds0 + ((it & 3) * 40 + blk) * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff), "s"(src + o) : "memory");
       }
-      off += MODE == 0 ? 384 * 32 : 40 * 1024;
+      off += MODE == 0 ? 384 * 32 : MODE == 3 ? 1536 * 32 : 40 * 1024;
       __builtin_amdgcn_s_waitcnt(0x0F70 | 5);      // all but the newest batch have landed
       __syncthreads();
     }
@@ -262,9 +265,10 @@ extern "C" int m2_probe_l2_stream_fwd(int mode, int iters, const void* region, l
                                       void* stream) {
   if (!region || !sink || iters <= 0) return set_error(M2_ERR_ARG, "m2_probe_l2_stream_fwd: null pointer or non-positive iters");
   if (region_bytes < (1 << 20)) return set_error(M2_ERR_ARG, "m2_probe_l2_stream_fwd: region of %ld bytes, need at least 1 MiB", region_bytes);
-  if (mode < 0 || mode > 2) return set_error(M2_ERR_UNSUPPORTED, "m2_probe_l2_stream_fwd: mode must be 0, 1 or 2");
+  if (mode < 0 || mode > 3) return set_error(M2_ERR_UNSUPPORTED, "m2_probe_l2_stream_fwd: mode must be 0 .. 3");
   const int lds = 160 * 1024;
-  auto kern = mode == 0 ? probe_l2_stream_kernel<0> : mode == 1 ? probe_l2_stream_kernel<1> : probe_l2_stream_kernel<2>;
+  auto kern = mode == 0 ? probe_l2_stream_kernel<0> : mode == 1 ? probe_l2_stream_kernel<1> : mode == 2 ? probe_l2_stream_kernel<2>
+                        : probe_l2_stream_kernel<3>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(probe_l2_stream): %s", hipGetErrorString(e));
   if (workgroups) *workgroups = num_cus();
