@@ -213,13 +213,21 @@ def test_encoder_small(gpu, L, B, layers):
     out1, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
     e, e2 = rel_err(out1, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
-    # the whole MLP as one kernel, and the in-projection on this library's own GEMM kernel (options as well)
+    # the MLP as two kernels with an fp32 sum into the LayerNorm (the default is one kernel and a bf16 sum), and the
+    # in-projection on this library's own GEMM kernel
     for layer in model.encoder.layer:
         layer.mlp.fuse_wo_layernorm = False
-        layer.mlp.fuse_mlp = True
+        layer.mlp.fuse_mlp = False
+        layer.mlp.bf16_presum = False
         layer.attention.own_in_linear = True
     out2, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
     e, e2 = rel_err(out2, ref)
+    assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
+    # one kernel, fp32 sum
+    for layer in model.encoder.layer:
+        layer.mlp.fuse_mlp = True
+    out3, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
+    e, e2 = rel_err(out3, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
 
 
