@@ -100,8 +100,8 @@ int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, int nfilter
  * of a row is convolved on its own in polyphase form, again as two LDS-resident half transforms). */
 int m2_fftconv_supported_seqlen(int L);
 
-/* Bytes of the opaque spectrum buffer for d channels and sequence length L (both filters): 16 d L, and 24 d L at
- * L = 32768 (where each frequency pair also carries the odd-sample spectrum times its twiddle).  Always ask. */
+/* Bytes of the opaque spectrum buffer for d channels and sequence length L (both filters): 16 d L, the size of
+ * the four L-tap fp32 filters it is made from.  Always ask. */
 size_t m2_filter_spectrum_bytes(int d, int L);
 
 /* taps1, taps2: (d, 2L) fp32 bidirectional taps of filter_fn and filter_fn2 (taps2 may be NULL:

@@ -383,7 +383,7 @@ extern "C" int m2_fftconv_supported_seqlen(int L) {
 }
 
 extern "C" size_t m2_filter_spectrum_bytes(int d, int L) {
-  if (L == 32768) return real_spectrum_bytes(d);      // (Ke, Ko, w Ko) per frequency pair and filter
+  if (L == 32768) return real_spectrum_bytes(d);      // (Ke, Ko) per frequency pair and filter: 16 d L as well
   return (size_t)d * (size_t)L * 16;        // d channels x 8 slots x (2L/16) work items x float4
 }
 

@@ -15,9 +15,10 @@
 // The H-point transform with a zero upper half is exactly what fft_split.h runs as two half transforms of
 // NS = H/2 = 16384 points (even and odd frequencies), and the pairing k <-> H - k is the mirror / complement
 // pairing of its last pass, so a thread holds both members of every pair.  Per pair the spectrum buffer
-// stores Ke, Ko and w_H^k Ko (24 bytes) in the order the multiply consumes them:
+// stores Ke and Ko (16 bytes) in the order the multiply consumes them; the root w_H^k is rebuilt in the multiply
+// from one per-thread constant per half transform and compile-time constants:
 //
-//   spec[channel][filter 0..1][half 0..1]{ float4 (Ke, Ko)[slot 0..15][T],  float2 (w Ko)[slot 0..15][T] }
+//   spec[channel][filter 0..1][half 0..1] float4 (Ke, Ko)[slot 0..15][T]
 //
 // The filter kernel gets Ke and Ko from ONE transform per filter: the (d, 2L) taps row read as H complex
 // numbers is k_even + i k_odd.
@@ -40,11 +41,14 @@
 namespace m2 {
 
 // One pair of the polyphase multiply: za = C[k], zb = C[H - k]; returns D[k] in za and D[H - k] in zb.
-// K = (Ke, Ko) and Kw = w_H^k Ko at frequency k, with the scale 1 / 4H folded in.
-__device__ __forceinline__ void pair_multiply_real(cf& za, cf& zb, float4 K, float2 Kw) {
+// K = (Ke, Ko) at frequency k, with the scale 1 / 4H folded in; the third factor w_H^k Ko is formed here: the root is
+// beta (this thread's group, one per half transform, the same for every row) times the constant w_64^S.
+template <int S>
+__device__ __forceinline__ void pair_multiply_real(cf& za, cf& zb, float4 K, cf beta) {
   const cf A = {za.re + zb.re, za.im - zb.im};         // 2 Ce
   const cf Bq = {za.im + zb.im, zb.re - za.re};        // 2 Co
-  const cf ke = {K.x, K.y}, ko = {K.z, K.w}, kw = {Kw.x, Kw.y};
+  const cf ke = {K.x, K.y}, ko = {K.z, K.w};
+  const cf kw = cmul(beta, mul_w64<S, false>(ko));
   const cf Ye = cadd(cmul(A, ke), cmul(Bq, kw));
   const cf Yo = cadd(cmul(A, ko), cmul(Bq, ke));
   za = {Ye.re - Yo.im, Ye.im + Yo.re};                 // Ye + i Yo
@@ -57,32 +61,29 @@ __device__ __forceinline__ cf self_multiply_real(cf z, float ke, float ko, float
 
 // spectral multiply of the 16 + 16 points a thread holds after fwd_groups, slots 4 HB .. 4 HB + 3 (same
 // pairing as multiply_batch in fft_split.h)
+// beta: root of the thread's group (slot s of it adds w_16^s); in the special work item of the even half the slots
+// 1 .. 7 belong to group 0 (root 1) and the slots 8 .. 15 to group R2 / 2 (root beta_sp, slot s - 8 of it).
 template <bool EVEN_SPECIAL, int HB>
-__device__ __forceinline__ void multiply_batch_real(cf (&x)[32], const float4 (&K)[4], const float2 (&W)[4]) {
+__device__ __forceinline__ void multiply_batch_real(cf (&x)[32], const float4 (&K)[4], cf beta, cf beta_sp) {
   static_for<0, 4>([&](auto ss) {
     constexpr int s = 4 * HB + decltype(ss)::value;
     const float4 k = K[decltype(ss)::value];
-    const float2 w = W[decltype(ss)::value];
     if constexpr (!EVEN_SPECIAL) {
-      pair_multiply_real(x[bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], k, w);
+      pair_multiply_real<4 * s>(x[bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], k, beta);
     } else if constexpr (s == 0) {
       // K = (Ke(0), Ko(0), Ke(H/2), Ko(H/2))
       x[bitrev(0, 4)] = self_multiply_real(x[bitrev(0, 4)], k.x, k.y, k.y);
       x[bitrev(8, 4)] = self_multiply_real(x[bitrev(8, 4)], k.z, k.w, -k.w);
     } else if constexpr (s < 8) {
-      pair_multiply_real(x[bitrev(s, 4)], x[bitrev(16 - s, 4)], k, w);
+      pair_multiply_real<4 * s>(x[bitrev(s, 4)], x[bitrev(16 - s, 4)], k, cf{1.f, 0.f});
     } else {
-      pair_multiply_real(x[16 + bitrev(s - 8, 4)], x[16 + bitrev(23 - s, 4)], k, w);
+      pair_multiply_real<4 * (s - 8)>(x[16 + bitrev(s - 8, 4)], x[16 + bitrev(23 - s, 4)], k, beta_sp);
     }
   });
 }
 template <int HB>
-__device__ __forceinline__ void load_spectrum_batch_real(float4 (&K)[4], float2 (&W)[4], const float4* __restrict__ sp4,
-                                                         const float2* __restrict__ sp2, int T) {
-  static_for<0, 4>([&](auto s) {
-    K[decltype(s)::value] = sp4[(4 * HB + decltype(s)::value) * T];
-    W[decltype(s)::value] = sp2[(4 * HB + decltype(s)::value) * T];
-  });
+__device__ __forceinline__ void load_spectrum_batch_real(float4 (&K)[4], const float4* __restrict__ sp4, int T) {
+  static_for<0, 4>([&](auto s) { K[decltype(s)::value] = sp4[(4 * HB + decltype(s)::value) * T]; });
 }
 
 // One half transform of one real signal: forward passes from registers (first-pass layout), polyphase multiply,
@@ -90,26 +91,25 @@ __device__ __forceinline__ void load_spectrum_batch_real(float4 (&K)[4], float2 
 // comes in four batches, each loaded while the one before it is multiplied.
 template <class P, bool ODD>
 __device__ __forceinline__ void half_convolution_real(cf (&x)[32], int t, float2* row, const float2* tab2,
-                                                      const cf (&b)[P::NB1], const float4* __restrict__ sp4,
-                                                      const float2* __restrict__ sp2, int ga, int gb, bool special) {
+                                                      const cf (&b)[P::NB1], const float4* __restrict__ sp4, cf beta,
+                                                      cf beta_sp, int ga, int gb, bool special) {
   fwd_pass1<P, ODD>(x, t, row, b);
   phase_barrier();
   fwd_pass2<P>(x, t, row, tab2);
   phase_barrier();
   float4 Ka[4], Kb[4];
-  float2 Wa[4], Wb[4];
-  load_spectrum_batch_real<0>(Ka, Wa, sp4, sp2, P::T);
+  load_spectrum_batch_real<0>(Ka, sp4, P::T);
   fwd_groups<P>(x, row, ga, gb);
   __builtin_amdgcn_sched_barrier(0);
   auto multiply = [&](auto sp) __attribute__((always_inline)) {
     constexpr bool S = decltype(sp)::value == 1;
-    load_spectrum_batch_real<1>(Kb, Wb, sp4, sp2, P::T);
-    multiply_batch_real<S, 0>(x, Ka, Wa);
-    load_spectrum_batch_real<2>(Ka, Wa, sp4, sp2, P::T);
-    multiply_batch_real<S, 1>(x, Kb, Wb);
-    load_spectrum_batch_real<3>(Kb, Wb, sp4, sp2, P::T);
-    multiply_batch_real<S, 2>(x, Ka, Wa);
-    multiply_batch_real<S, 3>(x, Kb, Wb);
+    load_spectrum_batch_real<1>(Kb, sp4, P::T);
+    multiply_batch_real<S, 0>(x, Ka, beta, beta_sp);
+    load_spectrum_batch_real<2>(Ka, sp4, P::T);
+    multiply_batch_real<S, 1>(x, Kb, beta, beta_sp);
+    load_spectrum_batch_real<3>(Kb, sp4, P::T);
+    multiply_batch_real<S, 2>(x, Ka, beta, beta_sp);
+    multiply_batch_real<S, 3>(x, Kb, beta, beta_sp);
   };
   if (!ODD && special) multiply(ic<1>{});
   else multiply(ic<0>{});
@@ -121,9 +121,9 @@ __device__ __forceinline__ void half_convolution_real(cf (&x)[32], int t, float2
   inv_pass1<P, ODD>(x, t, row, b);
 }
 
-// floats of the spectrum buffer per (channel, filter, half): 16 slots x T work items x (float4 + float2)
+// floats of the spectrum buffer per (channel, filter, half): 16 slots x T work items x float4
 template <class P>
-constexpr long real_spec_block() { return 16L * P::T * 6; }
+constexpr long real_spec_block() { return 16L * P::T * 4; }
 
 // ------------------------------------------------------------------------------------------
 // global memory in first-pass layout: complex slot m <-> time steps 2m, 2m + 1
@@ -238,6 +238,11 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
   cf b[P::NB1];
   static_for<0, P::NB1>([&](auto ii) { b[decltype(ii)::value] = unit_root(t + T * decltype(ii)::value, P::N); });
   const SplitGroups<P> grp = split_groups<P>(t);
+  // roots of the polyphase multiply: frequency k = k0 + R1 R2 s for slot s of group g, k0 = g / R2 + R1 (g % R2), and
+  // the pair at k of the half transform sits at 2 k + ODD of the H-point transform
+  const cf beta_e = unit_root(2 * (grp.ge / P::R2 + P::R1 * (grp.ge % P::R2)), P::N);
+  const cf beta_o = unit_root(2 * (grp.go / P::R2 + P::R1 * (grp.go % P::R2)) + 1, P::N);
+  const cf beta_sp = unit_root(2 * (P::R1 * (P::R2 / 2)), P::N);
   phase_barrier();
 
   // workgroup -> (channel, batch row) as in mixer_split_kernel: XCD e takes the channels c = e (mod 8)
@@ -270,8 +275,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
     static_for<0, 32>([&](auto rr) { acc[decltype(rr)::value] = x[decltype(rr)::value]; });     // a, for the odd half
     {
       const float4* sp4 = reinterpret_cast<const float4*>(spc) + t;
-      const float2* sp2 = reinterpret_cast<const float2*>(spc + 64L * T) + t;
-      half_convolution_real<P, false>(x, t, row, tab2, b, sp4, sp2, grp.ge, grp.gm, grp.special);
+      half_convolution_real<P, false>(x, t, row, tab2, b, sp4, beta_e, beta_sp, grp.ge, grp.gm, grp.special);
     }
     static_for<0, 32>([&](auto rr) {       // x <- a for the odd half, acc <- the even half's result
       constexpr int r = decltype(rr)::value;
@@ -281,8 +285,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
     });
     {
       const float4* sp4 = reinterpret_cast<const float4*>(spc + BLK) + t;
-      const float2* sp2 = reinterpret_cast<const float2*>(spc + BLK + 64L * T) + t;
-      half_convolution_real<P, true>(x, t, row, tab2, b, sp4, sp2, grp.go, grp.gc, false);
+      half_convolution_real<P, true>(x, t, row, tab2, b, sp4, beta_o, beta_sp, grp.go, grp.gc, false);
     }
     static_for<0, 32>([&](auto rr) {
       constexpr int r = decltype(rr)::value;
@@ -310,8 +313,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
       load_slots<P, float>(pu, t, x);
       {
         const float4* sp4 = reinterpret_cast<const float4*>(spc + 2 * BLK) + t;
-        const float2* sp2 = reinterpret_cast<const float2*>(spc + 2 * BLK + 64L * T) + t;
-        half_convolution_real<P, false>(x, t, row, tab2, b, sp4, sp2, grp.ge, grp.gm, grp.special);
+        half_convolution_real<P, false>(x, t, row, tab2, b, sp4, beta_e, beta_sp, grp.ge, grp.gm, grp.special);
       }
       static_for<0, 32>([&](auto rr) {
         constexpr int r = decltype(rr)::value;
@@ -323,8 +325,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
       load_slots<P, float>(pu + again, t, x);
       {
         const float4* sp4 = reinterpret_cast<const float4*>(spc + 3 * BLK) + t;
-        const float2* sp2 = reinterpret_cast<const float2*>(spc + 3 * BLK + 64L * T) + t;
-        half_convolution_real<P, true>(x, t, row, tab2, b, sp4, sp2, grp.go, grp.gc, false);
+        half_convolution_real<P, true>(x, t, row, tab2, b, sp4, beta_o, beta_sp, grp.go, grp.gc, false);
       }
       static_for<0, 32>([&](auto rr) {
         constexpr int r = decltype(rr)::value;
@@ -342,7 +343,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
 }
 
 // ------------------------------------------------------------------------------------------
-// filter taps -> (Ke, Ko, w Ko) in the layout above; work item = (channel, filter), both half transforms
+// filter taps -> (Ke, Ko) in the layout above; work item = (channel, filter), both half transforms
 // ------------------------------------------------------------------------------------------
 template <class P>
 __global__ __launch_bounds__(P::T) void filter_spectrum_real_kernel(
@@ -376,12 +377,7 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_real_kernel(
     if (!taps) {
       static_for<0, 2>([&](auto hh) {
         float4* z4 = reinterpret_cast<float4*>(blk + decltype(hh)::value * BLK) + t;
-        float2* z2 = reinterpret_cast<float2*>(blk + decltype(hh)::value * BLK + 64L * T) + t;
-        static_for<0, 16>([&](auto ss) {
-          constexpr int s = decltype(ss)::value;
-          z4[s * T] = make_float4(0.f, 0.f, 0.f, 0.f);
-          z2[s * T] = make_float2(0.f, 0.f);
-        });
+        static_for<0, 16>([&](auto ss) { z4[decltype(ss)::value * T] = make_float4(0.f, 0.f, 0.f, 0.f); });
       });
       continue;
     }
@@ -408,7 +404,6 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_real_kernel(
     auto one_half = [&](auto hh) __attribute__((always_inline)) {
       constexpr bool ODD = decltype(hh)::value == 1;
       float4* sp4 = reinterpret_cast<float4*>(blk + (ODD ? BLK : 0)) + t;
-      float2* sp2 = reinterpret_cast<float2*>(blk + (ODD ? BLK : 0) + 64L * T) + t;
       if constexpr (ODD) {
         static_for<0, Q>([&](auto qq) {
           constexpr int q = decltype(qq)::value;
@@ -428,37 +423,26 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_real_kernel(
       fwd_groups<P>(x, row, ga, gb);
       __syncthreads();      // LDS is restaged by the next half / item
 
-      // (Ke, Ko) of the pair (za at frequency k of this half transform, zb at its partner), and w_H^kk Ko with
-      // kk = 2 k + ODD the frequency of za in the H-point transform.  k = k0 + R1 R2 s for slot s of a group,
-      // so the root is w_H^(2 k0 + ODD) (one sincos per group) times the constant w_16^s.
-      auto emit = [&](auto ss, auto slot, cf za, cf zb, cf beta) __attribute__((always_inline)) {
-        constexpr int s = decltype(ss)::value;
-        const cf ke = {scale * (za.re + zb.re), scale * (za.im - zb.im)};
-        const cf ko = {scale * (za.im + zb.im), scale * (zb.re - za.re)};
-        const cf kw = cmul(beta, mul_w64<4 * s, false>(ko));
-        sp4[decltype(slot)::value * T] = make_float4(ke.re, ke.im, ko.re, ko.im);
-        sp2[decltype(slot)::value * T] = make_float2(kw.re, kw.im);
+      // (Ke, Ko) of the pair (za at frequency k of this half transform, zb at its partner)
+      auto emit = [&](auto slot, cf za, cf zb) __attribute__((always_inline)) {
+        sp4[decltype(slot)::value * T] = make_float4(scale * (za.re + zb.re), scale * (za.im - zb.im),
+                                                     scale * (za.im + zb.im), scale * (zb.re - za.re));
       };
       if (!ODD && grp.special) {
         const cf z0 = x[bitrev(0, 4)], zn = x[bitrev(8, 4)];
         sp4[0] = make_float4(4.f * scale * z0.re, 4.f * scale * z0.im, 4.f * scale * zn.re, 4.f * scale * zn.im);
-        sp2[0] = make_float2(0.f, 0.f);
-        const cf one = {1.f, 0.f};                                  // group 0: k0 = 0
         static_for<1, 8>([&](auto ss) {
           constexpr int s = decltype(ss)::value;
-          emit(ss, ss, x[bitrev(s, 4)], x[bitrev(16 - s, 4)], one);
+          emit(ss, x[bitrev(s, 4)], x[bitrev(16 - s, 4)]);
         });
-        const cf beta = unit_root(2 * (R1 * (R2 / 2)), H);          // group R2/2: k0 = R1 R2 / 2
         static_for<0, 8>([&](auto ss) {
           constexpr int s = decltype(ss)::value;
-          emit(ss, ic<8 + s>{}, x[16 + bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], beta);
+          emit(ic<8 + s>{}, x[16 + bitrev(s, 4)], x[16 + bitrev(15 - s, 4)]);
         });
       } else {
-        const int k0 = ga / R2 + R1 * (ga % R2);                    // frequency of slot 0 of group ga
-        const cf beta = unit_root(2 * k0 + (ODD ? 1 : 0), H);
         static_for<0, 16>([&](auto ss) {
           constexpr int s = decltype(ss)::value;
-          emit(ss, ss, x[bitrev(s, 4)], x[16 + bitrev(15 - s, 4)], beta);
+          emit(ss, x[bitrev(s, 4)], x[16 + bitrev(15 - s, 4)]);
         });
       }
     };
