@@ -234,14 +234,31 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int s = 0; s < kFKS; ++s) asm volatile("" : "+v"(xa[s]), "+v"(xb[s]));
 
     // Iteration i = 0 .. nchunks of the tile.  Iteration 0 has no previous chunk (gelu * value of zeros is zero, the
-    // second product adds nothing); iteration nchunks repeats the first products of the last chunk for nothing: both
-    // keep the loop body free of branches at 1 / nchunks more MFMAs.
-    for (int i = 0; i <= nchunks; ++i, ++n) {
+    // second product adds nothing: that keeps the body free of branches).  Iteration nchunks has no chunk of its own:
+    // it is a second copy of the body (TAIL) without the first products, which first requests what the end of the tile
+    // needs -- the next tile's x rows into the registers that have just become free, and this tile's residual rows --
+    // so that those loads travel while the last second product runs.
+    const int row = tile * kFRows + 16 * wave + i16;
+    const int rowc = row < M ? row : M - 1;
+    const long o0 = (long)rowc * d + r * kFP + 4 * q4;
+    u32x2 rres[12];
+    auto iteration = [&](auto tail_) __attribute__((always_inline)) {
+      constexpr bool TAIL = decltype(tail_)::value;
+      if constexpr (TAIL) {
+        if (tile + tile_step < ntiles) load_x(tile + tile_step);
+        if (resid) {
+          static_for<0, 12>([&](auto tt) {
+            rres[decltype(tt)::value] = *reinterpret_cast<const u32x2*>(resid + o0 + 16 * decltype(tt)::value);
+          });
+        }
+      }
       float gl[8];
       static_for<0, kNM>([&](auto kk) {
         constexpr int k = decltype(kk)::value;
         const bf16x8 a = __builtin_bit_cast(bf16x8, ring[k % kPF]);
-        if constexpr (k < 24) {
+        if constexpr (k < 24 && TAIL) {
+          // nothing to multiply; the operand read below still refills the ring for the next iteration
+        } else if constexpr (k < 24) {
           constexpr int s = k / 4, sel = k % 4, t = sel >> 1, val = sel & 1;
           floatx4& acc = val ? v[t] : g[t];
           if constexpr (s == 0) {
@@ -286,16 +303,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       else __builtin_amdgcn_s_waitcnt(kWaitVmBatch1);
       __syncthreads();
       __builtin_amdgcn_sched_barrier(0);
-    }
+      ++n;
+    };
+    for (int i = 0; i < nchunks; ++i) iteration(ic<0>{});
+    iteration(ic<1>{});
 
-    // ---- end of the tile: the next tile's x rows are requested first, then this tile's results leave.
+    // ---- end of the tile: this tile's results leave.
     // Accumulator element j of tile tau is output column 16 tau + 4 q + j of x-row n.
-    const int row = tile * kFRows + 16 * wave + i16;
     tile += tile_step;
     const bool more = tile < ntiles;
-    if (more) load_x(tile);
     if (row < M) {
-      const long o0 = (long)row * d + r * kFP + 4 * q4;
       static_for<0, 12>([&](auto tt) {
         constexpr int t = decltype(tt)::value;
         float4 val = make_float4(acc_out[t][0], acc_out[t][1], acc_out[t][2], acc_out[t][3]);
@@ -304,7 +321,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           val.x += bq.x; val.y += bq.y; val.z += bq.z; val.w += bq.w;
         }
         if (resid) {
-          const uint2 rr = *reinterpret_cast<const uint2*>(resid + o0 + 16 * t);
+          const u32x2 rr = rres[t];
           val.x += __uint_as_float(rr.x << 16); val.y += __uint_as_float(rr.x & 0xffff0000u);
           val.z += __uint_as_float(rr.y << 16); val.w += __uint_as_float(rr.y & 0xffff0000u);
         }
