@@ -226,24 +226,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     static_for<0, 12>([&](auto tt) {
       static_for<0, 4>([&](auto vv) { acc_out[decltype(tt)::value][decltype(vv)::value] = 0.f; });
     });
-    static_for<0, 8>([&](auto ee) { gp[decltype(ee)::value] = 0.f; vp[decltype(ee)::value] = 0.f; });
     // The x loads complete here, once per tile: consumed before the loop, the compiler has no reason to keep a
     // "load may be pending" mark on the x registers around the loop's back edge (that would put a full
     // vector-memory wait, which also waits for the direct-to-LDS loads just issued, into every iteration).
 #pragma unroll
     for (int s = 0; s < kFKS; ++s) asm volatile("" : "+v"(xa[s]), "+v"(xb[s]));
 
-    // Iteration i = 0 .. nchunks of the tile.  Iteration 0 has no previous chunk (gelu * value of zeros is zero, the
-    // second product adds nothing: that keeps the body free of branches).  Iteration nchunks has no chunk of its own:
-    // it is a second copy of the body (TAIL) without the first products, which first requests what the end of the tile
-    // needs -- the next tile's x rows into the registers that have just become free, and this tile's residual rows --
-    // so that those loads travel while the last second product runs.
+    // Iteration i = 0 .. nchunks of the tile, in three copies of one body.  Iteration 0 (HEAD) has no previous chunk:
+    // no gelu * value, no second product.  Iteration nchunks (TAIL) has no chunk of its own: no first products; it
+    // first requests what the end of the tile needs -- the next tile's x rows into the registers that have just become
+    // free, and this tile's residual rows -- so that those loads travel while the last second product runs.
     const int row = tile * kFRows + 16 * wave + i16;
     const int rowc = row < M ? row : M - 1;
     const long o0 = (long)rowc * d + r * kFP + 4 * q4;
     u32x2 rres[12];
-    auto iteration = [&](auto tail_) __attribute__((always_inline)) {
-      constexpr bool TAIL = decltype(tail_)::value;
+    auto iteration = [&](auto which_) __attribute__((always_inline)) {
+      constexpr bool TAIL = decltype(which_)::value == 1, HEAD = decltype(which_)::value == 2;
       if constexpr (TAIL) {
         if (tile + tile_step < ntiles) load_x(tile + tile_step);
         if (resid) {
@@ -267,7 +265,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           } else {
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, val ? xb[s] : xa[s], acc, 0, 0, 0);
           }
-        } else {
+        } else if constexpr (!HEAD) {
           acc_out[k - 24] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, gt, acc_out[k - 24], 0, 0, 0);
         }
         // next operand: this iteration's while k + kPF < 36, else the next iteration's
@@ -280,8 +278,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if constexpr (k % 7 == 1 && k / 7 < kFBatch) dma_one(n + 3, it3, ic<k / 7>{});
         // vector-ALU work riding along: gelu * value of the previous chunk (one element per 3 MFMAs of the first
         // products), then its packing; during the second product the accumulators just finished are copied out
-        if constexpr (k < 24 && k % 3 == 0) gl[k / 3] = gelu_erf_poly(gp[k / 3]) * vp[k / 3];
-        if constexpr (k == 23) {
+        if constexpr (k < 24 && k % 3 == 0 && !HEAD) gl[k / 3] = gelu_erf_poly(gp[k / 3]) * vp[k / 3];
+        if constexpr (k == 23 && !HEAD) {
           u32x4 pk;
           pk.x = pack_bf16x2(gl[0], gl[1]);
           pk.y = pack_bf16x2(gl[2], gl[3]);
@@ -305,7 +303,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       __builtin_amdgcn_sched_barrier(0);
       ++n;
     };
-    for (int i = 0; i < nchunks; ++i) iteration(ic<0>{});
+    iteration(ic<2>{});
+    for (int i = 1; i < nchunks; ++i) iteration(ic<0>{});
     iteration(ic<1>{});
 
     // ---- end of the tile: this tile's results leave.
