@@ -125,6 +125,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     OUT* __restrict__ out,                // (M, 768)
     int M, int I, int ntiles) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ __attribute__((aligned(16))) float bias_s[kFP];      // this r's slice of the bias, read at every tile's end
   const int tid = threadIdx.x, lane = tid & 63, i16 = lane & 15, q4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): XCD e works on output block r = e % 4 only,
@@ -139,6 +140,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int nchunks = IS / kFChunk;
   const int gb = r >> 1;                  // gate block; the value block is gb + 2
   const int d = 4 * kFP;
+  if (tid < kFP) bias_s[tid] = bias ? bias[r * kFP + tid] : 0.f;      // visible after the prologue's barrier
 
   // ---- the wave's x rows as stationary B operands: lane (n, q) holds x[row n][32 s + 8 q .. + 8) of both blocks
   bf16x8 xa[kFKS], xb[kFKS];
@@ -315,8 +317,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       static_for<0, 12>([&](auto tt) {
         constexpr int t = decltype(tt)::value;
         float4 val = make_float4(acc_out[t][0], acc_out[t][1], acc_out[t][2], acc_out[t][3]);
-        if (bias) {
-          const float4 bq = *reinterpret_cast<const float4*>(bias + r * kFP + 4 * q4 + 16 * t);
+        {
+          const float4 bq = *reinterpret_cast<const float4*>(bias_s + 4 * q4 + 16 * t);
           val.x += bq.x; val.y += bq.y; val.z += bq.z; val.w += bq.w;
         }
         if (resid) {
