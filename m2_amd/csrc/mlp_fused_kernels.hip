@@ -220,14 +220,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int kPF = 12;      // divides kNM, so that operand k of every iteration sits in ring slot k % kPF
   static_assert(kNM % kPF == 0, "the ring must close over an iteration");
   const unsigned char* lane_base = smem + 16 * lane;
-  auto operand_addr = [&](int n, auto kk) __attribute__((always_inline)) -> const unsigned char* {
+  // Operand k of an iteration sits at a compile-time offset from one of two addresses (the lane's 16 bytes in the
+  // iteration's Wg / Wv stage and in its Wo stage); the four addresses an iteration uses (its own and the next
+  // iteration's) are formed once at its top, so that an operand read is one LDS instruction and nothing else.
+  auto operand_off = [&](auto kk) constexpr -> int {
     constexpr int k = decltype(kk)::value;
     if constexpr (k < 24) {
       constexpr int s = k / 4, sel = k % 4, t = sel >> 1, val = sel & 1;
-      return lane_base + stage_gv(n) + ((2 * val + t) * kFKS + s) * kFBlk;
+      return ((2 * val + t) * kFKS + s) * kFBlk;
     } else {
-      return lane_base + stage_wo(n) + (k - 24) * kFBlk;
+      return (k - 24) * kFBlk;
     }
+  };
+  auto operand_addr = [&](int n, auto kk) __attribute__((always_inline)) -> const unsigned char* {
+    constexpr int k = decltype(kk)::value;
+    return lane_base + (k < 24 ? stage_gv(n) : stage_wo(n)) + operand_off(kk);
   };
   u32x4 ring[kPF];
   bf16x8 gt;
@@ -276,6 +283,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
       }
       float gl[8];
+      unsigned ogv0 = 16 * lane + stage_gv(n), owo0 = 16 * lane + stage_wo(n);
+      unsigned ogv1 = 16 * lane + stage_gv(n + 1), owo1 = 16 * lane + stage_wo(n + 1);
+      asm volatile("" : "+v"(ogv0), "+v"(owo0), "+v"(ogv1), "+v"(owo1));
       static_for<0, kNM>([&](auto kk) {
         constexpr int k = decltype(kk)::value;
         const bf16x8 a = __builtin_bit_cast(bf16x8, ring[k % kPF]);
@@ -294,8 +304,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           acc_out[k - 24] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, gt, acc_out[k - 24], 0, 0, 0);
         }
         // next operand: this iteration's while k + kPF < 36, else the next iteration's
-        if constexpr (k + kPF < kNM) ring[k % kPF] = *reinterpret_cast<const u32x4*>(operand_addr(n, ic<k + kPF>{}));
-        else ring[k % kPF] = *reinterpret_cast<const u32x4*>(operand_addr(n + 1, ic<k + kPF - kNM>{}));
+        if constexpr (k + kPF < kNM)
+          ring[k % kPF] = *reinterpret_cast<const u32x4*>(smem + (k + kPF < 24 ? ogv0 : owo0) + operand_off(ic<k + kPF>{}));
+        else
+          ring[k % kPF] = *reinterpret_cast<const u32x4*>(smem + (k + kPF - kNM < 24 ? ogv1 : owo1) + operand_off(ic<k + kPF - kNM>{}));
         // The batch of direct loads for iteration n + 3, one load every seventh MFMA: Wg / Wv into the stage last
         // read in iteration n - 1, Wo into the one last read in iteration n - 1 as well, both before the barrier that
         // started this iteration.  (Issued together at the top, the loads of the workgroup fill the memory
