@@ -151,13 +151,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   __shared__ __attribute__((aligned(16))) float bias_s[kFP];      // this r's slice of the bias, read at every tile's end
   const int tid = threadIdx.x, lane = tid & 63, i16 = lane & 15, q4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): XCD e works on output block r = e % 4 only,
-  // so its L2 holds one quarter of the weights, and on the row tiles of parity e / 4.  A workgroup is persistent:
-  // it walks over its row tiles while the weight stream through LDS just keeps cycling.
-  const int xcd = blockIdx.x & 7;
-  const int r = xcd & 3;
+  // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): XCD e works on the two output blocks
+  // r = 2 (e % 2), 2 (e % 2) + 1, which are fed by the same two blocks of x, and on the row tiles = e / 2 (mod 4);
+  // neighbouring workgroups of an XCD take the same row tile with the two r, so its L2 holds half of the weights
+  // and the second read of a tile's x rows hits it.  A workgroup is persistent: it walks over its row tiles while
+  // the weight stream through LDS just keeps cycling.  (The grid has an even number of workgroups per XCD.)
+  const int xcd = blockIdx.x & 7, slot = (int)(blockIdx.x >> 3);
+  const int r = 2 * (xcd & 1) + (slot & 1);
   const int tile_step = 2 * (int)(gridDim.x >> 3);
-  int tile = 2 * (int)(blockIdx.x >> 3) + (xcd >> 2);
+  int tile = 4 * (slot >> 1) + (xcd >> 1);
   if (tile >= ntiles) return;
   const int IS = I >> 2;                  // gated columns of this r
   const int nchunks = IS / kFChunk;
@@ -431,8 +433,8 @@ extern "C" int m2_mlp_fused_fwd(const void* x, const void* w_packed, const float
                      nblocks, in_features, intermediate);
   const int ntiles = (M + kFRows - 1) / kFRows;
   // one persistent workgroup per compute unit (144 KB of LDS each), 8 per step so that every XCD gets its share
-  int per_xcd = num_cus() / 8;
-  if (per_xcd > (ntiles + 1) / 2) per_xcd = (ntiles + 1) / 2;
+  int per_xcd = (num_cus() / 8) & ~1;
+  if (per_xcd > 2 * ((ntiles + 3) / 4)) per_xcd = 2 * ((ntiles + 3) / 4);
   const dim3 grid(8 * per_xcd);
   hipStream_t st = (hipStream_t)stream;
   if (out_dtype == M2_DTYPE_F32) {
