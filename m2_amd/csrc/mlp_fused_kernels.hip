@@ -115,9 +115,11 @@ __device__ __forceinline__ void load_to_lds(unsigned lds, unsigned voff, const v
 // Re-packs gated_layers.weight (4, I / 2, 192) and wo.weight (4, 192, I / 4) into the image of the LDS stages: for
 // r = 0 .. 3 and chunk c (32 gated columns) 24 Wg / Wv blocks and 12 Wo blocks of 64 lanes x 16 bytes.  One thread
 // per 16-byte piece.  Lane (i, q) of Wg / Wv block ((value, t), s) holds row gamma(16 t + i) = 8 (i / 4) + 4 t + i % 4
-// of the chunk, K = 32 s + 8 q .. + 7; of Wo block tau the row of output column 48 (i / 4) + 4 tau + i % 4, K = 8 q .. + 7
-// of the chunk (with that order of the output columns a lane of the main kernel ends up with 48 consecutive
-// columns of its row, which leave in 16-byte pieces).
+// of the chunk, K = 32 s + 8 q .. + 7; of Wo block tau the row of output column 32 (tau / 2) + 8 (i / 4) + 4 (tau % 2) + i % 4,
+// K = 8 q .. + 7 of the chunk.  With that order of the output columns lane (n, q) of the main kernel ends up with the
+// columns 32 s + 8 q .. + 7 (s = 0 .. 5) of its row: they leave as six 16-byte pieces, and the four lanes of a row
+// write 64 contiguous bytes per store instruction (48 consecutive columns per lane, i.e. four pieces 96 bytes
+// apart per instruction, cost 26 us of stores per launch at M = 32768).
 __global__ __launch_bounds__(256) void mlp_fused_pack_kernel(const uint16_t* __restrict__ wg, const uint16_t* __restrict__ wo,
                                                              u32x4* __restrict__ packed, int I) {
   const int IS = I >> 2, q = I >> 1, nchunks = IS / kFChunk;
@@ -134,7 +136,8 @@ __global__ __launch_bounds__(256) void mlp_fused_pack_kernel(const uint16_t* __r
     const int gamma = 8 * (i16 >> 2) + 4 * t + (i16 & 3);
     src = wg + (((long)((r >> 1) + 2 * val) * q + (long)(r & 1) * IS + c * kFChunk + gamma) * kFP + 32 * s + 8 * q4);
   } else {
-    src = wo + (((long)r * kFP + 48 * (i16 >> 2) + 4 * (blk - 24) + (i16 & 3)) * IS + c * kFChunk + 8 * q4);
+    const int tau = blk - 24;
+    src = wo + (((long)r * kFP + 32 * (tau >> 1) + 8 * (i16 >> 2) + 4 * (tau & 1) + (i16 & 3)) * IS + c * kFChunk + 8 * q4);
   }
   packed[piece] = *reinterpret_cast<const u32x4*>(src);
 }
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   // ---- staging.  The packed weights hold, per (r, chunk), 36 operand blocks of 1 KB, lane-major: Wg / Wv block
   // ((value, row tile t), K step s) = index (2 value + t) 6 + s, then Wo blocks tau = 0 .. 11 (the output
-  // columns 48 (i / 4) + 4 tau + i % 4, i < 16); lane (i, q) of a block holds what lane (i, q) of the MFMA needs.  Wave w copies the Wg / Wv blocks
+  // columns 32 (tau / 2) + 8 (i / 4) + 4 (tau % 2) + i % 4, i < 16); lane (i, q) of a block holds what lane (i, q) of the MFMA needs.  Wave w copies the Wg / Wv blocks
   // w, w + 8, w + 16, the Wo block w and, for w < 4, the Wo block w + 8.
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
   const unsigned voff = 16 * lane;
@@ -272,15 +275,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // free, and this tile's residual rows -- so that those loads travel while the last second product runs.
     const int row = tile * kFRows + 16 * wave + i16;
     const int rowc = row < M ? row : M - 1;
-    const long o0 = (long)rowc * d + r * kFP + 48 * q4;
+    const long o0 = (long)rowc * d + r * kFP + 8 * q4;
     u32x4 rres[6];
     auto iteration = [&](auto which_) __attribute__((always_inline)) {
       constexpr bool TAIL = decltype(which_)::value == 1, HEAD = decltype(which_)::value == 2;
       if constexpr (TAIL) {
         if (tile + tile_step < ntiles) load_x(tile + tile_step);
+      }
+      if constexpr (HEAD) {
         if (resid) {
           static_for<0, 6>([&](auto mm) {
-            rres[decltype(mm)::value] = *reinterpret_cast<const u32x4*>(resid + o0 + 8 * decltype(mm)::value);
+            rres[decltype(mm)::value] = *reinterpret_cast<const u32x4*>(resid + o0 + 32 * decltype(mm)::value);
           });
         }
       }
@@ -357,7 +362,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     iteration(ic<1>{});
 
     // ---- end of the tile: this tile's results leave.  Accumulator element j of tile tau is output column
-    // 48 q + 4 tau + j of x-row n (the order the packed Wo rows were given): 48 consecutive columns per lane.
+    // 32 (tau / 2) + 8 q + 4 (tau % 2) + j of x-row n (the order the packed Wo rows were given): piece m of a lane =
+    // tiles 2 m and 2 m + 1 = the eight columns 32 m + 8 q .. + 7.
     tile += tile_step;
     const bool more = tile < ntiles;
     if (row < M) {
@@ -366,7 +372,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         float val[8];
         static_for<0, 8>([&](auto ee) {
           constexpr int e = decltype(ee)::value;
-          val[e] = acc_out[2 * m + e / 4][e % 4] + bias_s[48 * q4 + 8 * m + e];
+          val[e] = acc_out[2 * m + e / 4][e % 4] + bias_s[32 * m + 8 * q4 + e];
         });
         if (resid) {
           const u32x4 rr = rres[m];
@@ -381,10 +387,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           pk.y = pack_bf16x2(val[2], val[3]);
           pk.z = pack_bf16x2(val[4], val[5]);
           pk.w = pack_bf16x2(val[6], val[7]);
-          *reinterpret_cast<u32x4*>(out + o0 + 8 * m) = pk;
+          *reinterpret_cast<u32x4*>(out + o0 + 32 * m) = pk;
         } else {
-          *reinterpret_cast<float4*>(out + o0 + 8 * m) = make_float4(val[0], val[1], val[2], val[3]);
-          *reinterpret_cast<float4*>(out + o0 + 8 * m + 4) = make_float4(val[4], val[5], val[6], val[7]);
+          *reinterpret_cast<float4*>(out + o0 + 32 * m) = make_float4(val[0], val[1], val[2], val[3]);
+          *reinterpret_cast<float4*>(out + o0 + 32 * m + 4) = make_float4(val[4], val[5], val[6], val[7]);
         }
       });
     }
