@@ -75,7 +75,7 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
     // flight first; then short conv, gate, z = a + i u -> LDS
     GateRow<ACT, 4> gate;
     {
-      RawRow<ACT, 4> r1, r2, rv;
+      RawRow<ACT, 4, true> r1, r2, rv;      // the four accesses of a thread are consecutive
       f32x4_t ru[8];
       float w1[3], w2[3], wv[3], b1 = 0.f, b2 = 0.f, bv = 0.f, p1 = 0.f, p2 = 0.f, pv = 0.f;
       static_for<0, 4>([&](auto qq) {

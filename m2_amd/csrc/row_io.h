@@ -32,47 +32,63 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 // Raw registers of one access.  Kept as separate arrays of plain vectors (RawRow<ACT, Q>::a / b / h), not as
 // an array of structs: only the former are reliably promoted to registers.
-template <typename ACT, int Q> struct RawRow;
-template <int Q> struct RawRow<float, Q> {
+// CHAINED: the Q accesses are consecutive (access I starts where access I - 1 ends), so only access 0 fetches the
+// two elements before it; the others take them from the registers of their predecessor.
+template <typename ACT, int Q, bool CHAINED = false> struct RawRow;
+template <int Q, bool CHAINED> struct RawRow<float, Q, CHAINED> {
   f32x4_t a[Q], b[Q];
   f32x2_t h[Q];
   template <int I> __device__ __forceinline__ void fetch(const float* p, int n0) {
     a[I] = *reinterpret_cast<const f32x4_t*>(p + n0);
     b[I] = *reinterpret_cast<const f32x4_t*>(p + n0 + 4);
-    h[I] = *reinterpret_cast<const f32x2_t*>(p + (n0 > 0 ? n0 - 2 : 0));      // unused when n0 == 0
+    if constexpr (!(CHAINED && I > 0))
+      h[I] = *reinterpret_cast<const f32x2_t*>(p + (n0 > 0 ? n0 - 2 : 0));      // unused when n0 == 0
+  }
+  template <int I> __device__ __forceinline__ f32x2_t before() const {
+    if constexpr (CHAINED && I > 0) return f32x2_t{b[I - 1].z, b[I - 1].w};
+    else return h[I];
   }
   template <int I> __device__ __forceinline__ void expand(int n0, float add, float (&o)[10]) const {
-    o[0] = n0 > 0 ? h[I].x + add : 0.f;
-    o[1] = n0 > 0 ? h[I].y + add : 0.f;
+    const f32x2_t hh = before<I>();
+    o[0] = n0 > 0 ? hh.x + add : 0.f;
+    o[1] = n0 > 0 ? hh.y + add : 0.f;
     o[2] = a[I].x + add; o[3] = a[I].y + add; o[4] = a[I].z + add; o[5] = a[I].w + add;
     o[6] = b[I].x + add; o[7] = b[I].y + add; o[8] = b[I].z + add; o[9] = b[I].w + add;
   }
   // the same without the addend (no add instructions at all)
   template <int I> __device__ __forceinline__ void expand(int n0, float (&o)[10]) const {
-    o[0] = n0 > 0 ? h[I].x : 0.f;
-    o[1] = n0 > 0 ? h[I].y : 0.f;
+    const f32x2_t hh = before<I>();
+    o[0] = n0 > 0 ? hh.x : 0.f;
+    o[1] = n0 > 0 ? hh.y : 0.f;
     o[2] = a[I].x; o[3] = a[I].y; o[4] = a[I].z; o[5] = a[I].w;
     o[6] = b[I].x; o[7] = b[I].y; o[8] = b[I].z; o[9] = b[I].w;
   }
 };
-template <int Q> struct RawRow<uint16_t, Q> {
+template <int Q, bool CHAINED> struct RawRow<uint16_t, Q, CHAINED> {
   u32x4_t a[Q];
   uint32_t h[Q];
   template <int I> __device__ __forceinline__ void fetch(const uint16_t* p, int n0) {
     a[I] = *reinterpret_cast<const u32x4_t*>(p + n0);
-    h[I] = *reinterpret_cast<const uint32_t*>(p + (n0 > 0 ? n0 - 2 : 0));     // unused when n0 == 0
+    if constexpr (!(CHAINED && I > 0))
+      h[I] = *reinterpret_cast<const uint32_t*>(p + (n0 > 0 ? n0 - 2 : 0));     // unused when n0 == 0
+  }
+  template <int I> __device__ __forceinline__ uint32_t before() const {
+    if constexpr (CHAINED && I > 0) return a[I - 1].w;
+    else return h[I];
   }
   template <int I> __device__ __forceinline__ void expand(int n0, float add, float (&o)[10]) const {
-    o[0] = n0 > 0 ? __uint_as_float(h[I] << 16) + add : 0.f;
-    o[1] = n0 > 0 ? __uint_as_float(h[I] & 0xffff0000u) + add : 0.f;
+    const uint32_t hh = before<I>();
+    o[0] = n0 > 0 ? __uint_as_float(hh << 16) + add : 0.f;
+    o[1] = n0 > 0 ? __uint_as_float(hh & 0xffff0000u) + add : 0.f;
     o[2] = __uint_as_float(a[I].x << 16) + add; o[3] = __uint_as_float(a[I].x & 0xffff0000u) + add;
     o[4] = __uint_as_float(a[I].y << 16) + add; o[5] = __uint_as_float(a[I].y & 0xffff0000u) + add;
     o[6] = __uint_as_float(a[I].z << 16) + add; o[7] = __uint_as_float(a[I].z & 0xffff0000u) + add;
     o[8] = __uint_as_float(a[I].w << 16) + add; o[9] = __uint_as_float(a[I].w & 0xffff0000u) + add;
   }
   template <int I> __device__ __forceinline__ void expand(int n0, float (&o)[10]) const {
-    o[0] = n0 > 0 ? __uint_as_float(h[I] << 16) : 0.f;
-    o[1] = n0 > 0 ? __uint_as_float(h[I] & 0xffff0000u) : 0.f;
+    const uint32_t hh = before<I>();
+    o[0] = n0 > 0 ? __uint_as_float(hh << 16) : 0.f;
+    o[1] = n0 > 0 ? __uint_as_float(hh & 0xffff0000u) : 0.f;
     o[2] = __uint_as_float(a[I].x << 16); o[3] = __uint_as_float(a[I].x & 0xffff0000u);
     o[4] = __uint_as_float(a[I].y << 16); o[5] = __uint_as_float(a[I].y & 0xffff0000u);
     o[6] = __uint_as_float(a[I].z << 16); o[7] = __uint_as_float(a[I].z & 0xffff0000u);
