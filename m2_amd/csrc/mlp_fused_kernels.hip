@@ -30,8 +30,9 @@
 // laid out [operand block][lane]).  One barrier per chunk; the operand reads run ahead of the MFMAs through a ring
 // of registers that does not drain at the barrier (the next chunk is complete one barrier early).
 //
-// Every compute unit streams ALL weights of its r once per 128-row tile, from L2: 36 KB per 0.5 us of MFMA work, and
-// that stream, not the matrix pipe, is what bounds the kernel.  Measured on MI355X with all 256 compute units
+// Every compute unit streams ALL weights of its r once per 128-row tile, from L2: 36 KB per 0.5 us of MFMA work, more
+// than the L2 delivers to a compute unit at the MFMAs' pace (with that stream, the operand reads, the GELU and the
+// barrier, none of which hides behind the others, a chunk takes about 1.1 us).  Measured on MI355X with all 256 compute units
 // streaming (direct-to-LDS loads, L2 hits): 62 GB/s per compute unit when a load instruction covers 1 KB of
 // contiguous memory, 38 GB/s when it gathers sixteen 64-byte row pieces (the operand layout taken straight from the
 // row-major weights).  So the weights are re-packed once (m2_mlp_fused_pack) into the exact image of the LDS
