@@ -91,7 +91,7 @@ __device__ __forceinline__ void gelu_step(GeluChain& c, float x, float v, float&
 
 constexpr int kFP = 192;                    // block width of x and of the output (d / 4)
 constexpr int kFKS = kFP / 32;              // K steps of the first products (K = 32 per MFMA): 6
-constexpr int kFRows = 128;                 // rows per workgroup: 8 waves x 16
+constexpr int kFRows = 128;                 // rows per workgroup of 8 waves (16 per wave); the 4-wave variant for small M owns 64
 constexpr int kFChunk = 32;                 // gated columns per chunk
 constexpr int kFBlk = 1024;                 // one operand block: 64 lanes x 16 bytes = 16 rows x 32 K
 constexpr int kFGV = 2 * 2 * kFKS * kFBlk;  // Wg + Wv of a chunk: (gate | value) x 2 row tiles x 6 K steps = 24 KB
@@ -99,11 +99,10 @@ constexpr int kFWO = 12 * kFBlk;            // Wo of a chunk: 12 output tiles of
 constexpr int kFStages = 4;
 constexpr int kFLds = kFStages * (kFGV + kFWO);      // 144 KB
 constexpr int kFChunkBytes = kFGV + kFWO;   // a chunk in the packed weights: the image of its two stages
-constexpr int kFBatch = 5;                  // direct loads a wave issues per chunk: 3 (Wg / Wv) + 2 (Wo; 1 for waves 4 .. 7)
 
 // s_waitcnt immediates (vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8): wait for the vector-memory
 // counter only
-constexpr int kWaitVm0 = 0x0F70, kWaitVmBatch = 0x0F70 | kFBatch, kWaitVmBatch1 = 0x0F70 | (kFBatch - 1);
+constexpr int kWaitVm0 = 0x0F70;
 
 // One direct global -> LDS load: every lane fetches 16 bytes from base + voff, lane l's piece lands at LDS byte
 // address lds + 16 l.  Inline assembly on purpose: the compiler then neither tracks the LDS write (it would put a
@@ -143,8 +142,11 @@ __global__ __launch_bounds__(256) void mlp_fused_pack_kernel(const uint16_t* __r
   packed[piece] = *reinterpret_cast<const u32x4*>(src);
 }
 
-template <typename OUT>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mlp_fused_kernel(
+// WAVES = 8: the kernel as described above.  WAVES = 4: the same with workgroups of four waves and 64 rows, for row
+// counts at which 128-row tiles would leave compute units without work (M < 8192: one wave per SIMD, every wave
+// copies 9 of a chunk's 36 blocks).
+template <typename OUT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVES / 4, 2))) void mlp_fused_kernel(
     const uint16_t* __restrict__ x,       // (M, 768) bf16
     const unsigned char* __restrict__ wpk,      // both weights as packed by mlp_fused_pack_kernel
     const float* __restrict__ bias,       // (768) or null
@@ -174,7 +176,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // ---- the wave's x rows as stationary B operands: lane (n, q) holds x[row n][32 s + 8 q .. + 8) of both blocks
   bf16x8 xa[kFKS], xb[kFKS];
   auto load_x = [&](int t) __attribute__((always_inline)) {
-    int row = t * kFRows + 16 * wave + i16;
+    int row = t * (16 * WAVES) + 16 * wave + i16;
     row = row < M ? row : M - 1;
     const uint16_t* pa = x + (long)row * d + gb * kFP + 8 * q4;
     const uint16_t* pb = pa + 2 * kFP;
@@ -200,16 +202,29 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // Load j of the batch that feeds iteration n, which is iteration `it` (0 .. nchunks) of its tile: Wg / Wv of chunk
   // `it` (iteration nchunks only repeats the last chunk) or Wo of chunk it - 1 (iteration 0 multiplies zeros by
   // whatever finite numbers it finds: chunk 0).
+  constexpr int kBatch = 36 / WAVES + (36 % WAVES ? 1 : 0);      // loads per wave and chunk: 5 (8 waves) or 9 (4 waves)
+  constexpr int kGvLoads = 24 / WAVES;                             // of which Wg / Wv blocks: 3 or 6
+  constexpr int kDmaEvery = 36 / kBatch;                           // one load every 7th (4th) MFMA
   auto dma_one = [&](int n, int it, auto jj) __attribute__((always_inline)) {
     constexpr int j = decltype(jj)::value;
-    if constexpr (j < 3) {
+    if constexpr (j < kGvLoads) {
       const int cc = it < nchunks ? it : nchunks - 1;
-      load_to_lds(lds0 + stage_gv(n) + (wave + 8 * j) * kFBlk, voff, wr + (long)cc * kFChunkBytes + (wave + 8 * j) * kFBlk);
+      load_to_lds(lds0 + stage_gv(n) + (wave + WAVES * j) * kFBlk, voff, wr + (long)cc * kFChunkBytes + (wave + WAVES * j) * kFBlk);
     } else {
       const int cc = it > 0 ? it - 1 : 0;
-      const int tau = wave + 8 * (j - 3);
-      if (j == 3 || wave < 4)
+      const int tau = wave + WAVES * (j - kGvLoads);
+      if (WAVES * (j - kGvLoads + 1) <= 12 || wave < 12 - WAVES * (j - kGvLoads))      // the block exists
         load_to_lds(lds0 + stage_wo(n) + tau * kFBlk, voff, wr + (long)cc * kFChunkBytes + kFGV + tau * kFBlk);
+    }
+  };
+  // what a wave waits for before the barrier: everything but its newest batch (waves whose last Wo block does not
+  // exist issue one load fewer)
+  auto wait_batch = [&]() __attribute__((always_inline)) {
+    if constexpr (WAVES * (kBatch - kGvLoads) <= 12) {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | kBatch);
+    } else {
+      if (wave < 12 - WAVES * (kBatch - 1 - kGvLoads)) __builtin_amdgcn_s_waitcnt(0x0F70 | kBatch);
+      else __builtin_amdgcn_s_waitcnt(0x0F70 | (kBatch - 1));
     }
   };
 
@@ -248,7 +263,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // prologue: the batches of iterations 0 .. 2; then the ring for iteration 0
   int it3 = 0;             // which iteration of its tile iteration n + 3 is
   for (int n = 0; n < 3; ++n) {
-    static_for<0, kFBatch>([&](auto jj) { dma_one(n, it3, jj); });
+    static_for<0, kBatch>([&](auto jj) { dma_one(n, it3, jj); });
     it3 = it3 == nchunks ? 0 : it3 + 1;
   }
   __builtin_amdgcn_s_waitcnt(kWaitVm0);
@@ -274,7 +289,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // no gelu * value, no second product.  Iteration nchunks (TAIL) has no chunk of its own: no first products; it
     // first requests what the end of the tile needs -- the next tile's x rows into the registers that have just become
     // free, and this tile's residual rows -- so that those loads travel while the last second product runs.
-    const int row = tile * kFRows + 16 * wave + i16;
+    const int row = tile * (16 * WAVES) + 16 * wave + i16;
     const int rowc = row < M ? row : M - 1;
     const long o0 = (long)rowc * d + r * kFP + 8 * q4;
     u32x4 rres[6];
@@ -320,7 +335,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         // read in iteration n - 1, Wo into the one last read in iteration n - 1 as well, both before the barrier that
         // started this iteration.  (Issued together at the top, the loads of the workgroup fill the memory
         // pipeline's queue and every wave stalls behind its own loads: 21 us of 210 at M = 32768.)
-        if constexpr (k % 7 == 1 && k / 7 < kFBatch) dma_one(n + 3, it3, ic<k / 7>{});
+        if constexpr (k % kDmaEvery == 1 && k / kDmaEvery < kBatch) dma_one(n + 3, it3, ic<k / kDmaEvery>{});
         // vector-ALU work riding along: gelu * value of the previous chunk, all eight elements in one burst behind the
         // first MFMA (measured: one element after every third MFMA 151.7 us, two after every sixth 149.8, four after
         // every twelfth 149.4, all eight at once 147.3; four instructions after every MFMA 155.0), then its
@@ -352,8 +367,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       it3 = it3 == nchunks ? 0 : it3 + 1;
       // before the barrier: everything but this wave's newest batch has landed, so after the barrier the chunks of
       // iterations n + 1 and n + 2 are complete for everybody
-      if (wave < 4) __builtin_amdgcn_s_waitcnt(kWaitVmBatch);
-      else __builtin_amdgcn_s_waitcnt(kWaitVmBatch1);
+      wait_batch();
       __syncthreads();
       __builtin_amdgcn_sched_barrier(0);
       ++n;
@@ -405,6 +419,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 using namespace m2;
 
+template <typename OUT>
+static OUT* out_ptr(void (*)(const uint16_t*, const unsigned char*, const float*, const uint16_t*, OUT*, int, int, int));
+
 extern "C" int m2_mlp_fused_supported(int in_features, int intermediate, int nblocks) {
   return nblocks == 4 && in_features == 4 * kFP && intermediate > 0 && intermediate % (4 * kFChunk) == 0;
 }
@@ -438,24 +455,28 @@ extern "C" int m2_mlp_fused_fwd(const void* x, const void* w_packed, const float
                      "m2_mlp_fused_fwd: built for nblocks=4, in_features=768 and intermediate a multiple of 128 "
                      "(got nblocks=%d in=%d intermediate=%d); use m2_blockdiag_glu_fwd + m2_blockdiag_linear_fwd",
                      nblocks, in_features, intermediate);
-  const int ntiles = (M + kFRows - 1) / kFRows;
-  // one persistent workgroup per compute unit (144 KB of LDS each), 8 per step so that every XCD gets its share
+  // 128-row tiles and eight waves per workgroup; 64-row tiles and four waves where the 128-row tiles of the four
+  // output blocks would not occupy the compute units (M < 8192 on 256 of them)
+  const bool small = 4 * ((M + kFRows - 1) / kFRows) < num_cus();
+  const int rows = small ? kFRows / 2 : kFRows;
+  const int ntiles = (M + rows - 1) / rows;
+  // one persistent workgroup per compute unit (144 KB of LDS each), an even number per XCD
   int per_xcd = (num_cus() / 8) & ~1;
   if (per_xcd > 2 * ((ntiles + 3) / 4)) per_xcd = 2 * ((ntiles + 3) / 4);
   const dim3 grid(8 * per_xcd);
   hipStream_t st = (hipStream_t)stream;
-  if (out_dtype == M2_DTYPE_F32) {
-    auto kern = mlp_fused_kernel<float>;
+  auto launch = [&](auto kern, int threads) -> int {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kFLds);
     if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(mlp_fused): %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, grid, dim3(512), kFLds, st, (const uint16_t*)x, (const unsigned char*)w_packed,
-                       bias, (const uint16_t*)residual, (float*)out, M, intermediate, ntiles);
-  } else {
-    auto kern = mlp_fused_kernel<uint16_t>;
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kFLds);
-    if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(mlp_fused): %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, grid, dim3(512), kFLds, st, (const uint16_t*)x, (const unsigned char*)w_packed,
-                       bias, (const uint16_t*)residual, (uint16_t*)out, M, intermediate, ntiles);
-  }
+    hipLaunchKernelGGL(kern, grid, dim3(threads), kFLds, st, (const uint16_t*)x, (const unsigned char*)w_packed, bias,
+                       (const uint16_t*)residual, (decltype(out_ptr(kern)))out, M, intermediate, ntiles);
+    return 0;
+  };
+  int rc;
+  if (out_dtype == M2_DTYPE_F32)
+    rc = small ? launch(mlp_fused_kernel<float, 4>, 256) : launch(mlp_fused_kernel<float, 8>, 512);
+  else
+    rc = small ? launch(mlp_fused_kernel<uint16_t, 4>, 256) : launch(mlp_fused_kernel<uint16_t, 8>, 512);
+  if (rc) return rc;
   return check_launch("mlp_fused");
 }
