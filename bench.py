@@ -300,7 +300,7 @@ def main():
     for fn, tag in (("mixer_core", "mixer_core"), ("hyena_filter_taps", "filter_taps"),
                     ("filter_spectrum", "filter_spectrum"), ("blockdiag_glu", "blockdiag_glu"),
                     ("blockdiag_linear", "blockdiag_linear"), ("blockdiag_linear_layernorm", "wo_layernorm"),
-                    ("mlp_fused", "mlp_fused"),
+                    ("mlp_fused", "mlp_fused"), ("glu_stream", "glu_stream"),
                     ("layernorm", "layernorm"), ("embed_layernorm", "embed_layernorm")):
         wrapped[fn] = timer.wrap(ops, fn, tag)
 
@@ -317,7 +317,7 @@ def main():
         dt = time.perf_counter() - t0
     eager_ms = dt / args.steps * 1e3
     means = {tag: timer.mean_ms(tag) for tag in ("mixer_core", "filter_taps", "filter_spectrum", "blockdiag_glu",
-                                                  "blockdiag_linear", "wo_layernorm", "mlp_fused", "layernorm",
+                                                  "blockdiag_linear", "wo_layernorm", "mlp_fused", "glu_stream", "layernorm",
                                                   "embed_layernorm")
              if timer.count(tag)}
     n_core = timer.count("mixer_core")
@@ -383,13 +383,15 @@ def main():
               "ms_per_launch": t_mlp, "hbm_frac": mlp_bytes / (t_mlp * 1e-3) / 1e9 / HBM_PEAK_GBPS,
               "both_frac": mlp_tflops / MFMA_BF16_PEAK_TFLOPS}
     else:
-        t_glu = means["blockdiag_glu"]
+        # 384-wide blocks run the x-stationary kernel on packed weights (m2_glu_stream_fwd), others the tiled one
+        glu_entry = "m2_glu_stream_fwd" if "glu_stream" in means else "m2_blockdiag_glu_fwd"
+        t_glu = means["glu_stream"] if "glu_stream" in means else means["blockdiag_glu"]
         # the same kernels against the HBM roof: algorithmic bytes (bf16 in, fused GLU write; wo with its bf16
         # residual and fp32 sum) over the measured time, as a fraction of 8 TB/s
         glu_bytes = M * d * 2 + (2 * I * d // nbk) * 2 + M * I * 2
         wo_bytes = M * I * 2 + (I * d // nbk) * 2 + M * d * 2 + M * d * 4
         glu_tflops = glu_flops / (t_glu * 1e-3) / 1e12
-        k3 = {"kernel": "gated block-diagonal GEMM + GLU (m2_blockdiag_glu_fwd)", "bound": "mfma", "achieved": glu_tflops,
+        k3 = {"kernel": f"gated block-diagonal GEMM + GLU ({glu_entry})", "bound": "mfma", "achieved": glu_tflops,
               "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": glu_tflops / MFMA_BF16_PEAK_TFLOPS,
               "traffic": None, "flops_per_launch": glu_flops, "ms_per_launch": t_glu,
               "hbm_frac": glu_bytes / (t_glu * 1e-3) / 1e9 / HBM_PEAK_GBPS}

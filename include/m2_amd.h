@@ -193,6 +193,22 @@ int m2_mlp_fused_pack(const void* w_gated, const void* w_out, void* packed, int 
 int m2_mlp_fused_fwd(const void* x, const void* w_packed, const float* bias, const void* residual, void* out, int M,
                      int in_features, int intermediate, int nblocks, int out_dtype, void* stream);
 
+/* The gated block-diagonal GEMM with the GLU on its accumulators for 384-wide blocks, from packed weights:
+ * out (M, I) bf16 = gelu_erf(h[:, :I]) * h[:, I:], h = blockdiag_multiply(x, w_gated)  (bert/src/bert_layers.py:494-502,
+ * bert/src/mm/blockdiag_multiply.py:49-60).  Same arithmetic and result layout as m2_blockdiag_glu_fwd; the x rows stay
+ * in registers and the weights stream through LDS from a packed copy in which every 1 KB the kernel moves at a time is
+ * contiguous.  m2_glu_stream_pack writes that copy once per set of weights (w_gated (nblocks, 2I/nblocks,
+ * in/nblocks) bf16, gated_layers.weight; packed: m2_glu_stream_packed_bytes bytes of device memory, 16-byte aligned,
+ * the size of the weight).  m2_glu_stream_fwd: x (M, in_features) bf16, w_packed as written by m2_glu_stream_pack for
+ * the same shape, out (M, intermediate) bf16.  m2_glu_stream_supported returns 1 for the shapes the kernel is built for
+ * (nblocks == 4, in_features == 1536, intermediate % 128 == 0); for others m2_glu_stream_packed_bytes returns 0, the
+ * other two return M2_ERR_UNSUPPORTED and the caller uses m2_blockdiag_glu_fwd. */
+int m2_glu_stream_supported(int in_features, int intermediate, int nblocks);
+long m2_glu_stream_packed_bytes(int in_features, int intermediate, int nblocks);
+int m2_glu_stream_pack(const void* w_gated, void* packed, int in_features, int intermediate, int nblocks, void* stream);
+int m2_glu_stream_fwd(const void* x, const void* w_packed, void* out, int M, int in_features, int intermediate,
+                      int nblocks, void* stream);
+
 /* LayerNorm over the last dimension of x (M, d) fp32 (torch.nn.LayerNorm semantics, biased variance,
  * eps inside the root; bert/src/bert_layers.py:478-479,506 and :185-186,247).  Any of the three
  * outputs may be NULL: out_f32 (M, d) fp32, out_bf16 (M, d) bf16, out_channel_major (d, M) fp32 (the

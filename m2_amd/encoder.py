@@ -155,9 +155,25 @@ class BertGatedLinearUnitMLP(nn.Module):
                 self._packed = (wg, wo, ops.mlp_fused_pack(wg, wo))
             return ops.mlp_fused(a16, wg, wo, self.wo.bias.detach().float().contiguous(), a16, out_dtype=sum_dtype,
                                  packed=self._packed[2])
-        g = ops.blockdiag_glu(a16, self.gated_layers.weight_bf16())
+        g = self.glu(a16)
         return ops.blockdiag_linear(g, self.wo.weight_bf16(), self.wo.bias.detach().float().contiguous(), a16,
                                     out_dtype=sum_dtype)
+
+    # True: for 384-wide blocks (d = 1536, four blocks) the gated product + GLU runs as the kernel that keeps the x rows
+    # in registers and streams packed weights through LDS (m2_glu_stream_fwd) instead of the LDS-tiled GEMM with a GLU
+    # epilogue (m2_blockdiag_glu_fwd).  Same arithmetic; other shapes take the tiled kernel.
+    stream_glu = True
+    _packed_glu = None
+
+    def glu(self, a16: torch.Tensor) -> torch.Tensor:
+        """a16 (M, d) bf16 -> gelu(gate) * value of gated_layers(a16), (M, I) bf16."""
+        wg = self.gated_layers.weight_bf16()
+        if self.stream_glu and ops.glu_stream_supported(a16.shape[1], self.config.intermediate_size,
+                                                        self.config.monarch_mlp_nblocks):
+            if self._packed_glu is None or self._packed_glu[0] is not wg:      # rebuilt with the bf16 copy
+                self._packed_glu = (wg, ops.glu_stream_pack(wg))
+            return ops.glu_stream(a16, wg, packed=self._packed_glu[1])
+        return ops.blockdiag_glu(a16, wg)
 
     def ln_params(self):
         return self.layernorm.weight.detach().float(), self.layernorm.bias.detach().float(), self.layernorm.eps
@@ -170,7 +186,7 @@ class BertGatedLinearUnitMLP(nn.Module):
         w = self.wo.weight_bf16()
         nb, q, p = w.shape
         if self.fuse_wo_layernorm and ops.blockdiag_linear_layernorm_supported(nb * p, nb * q, nb):
-            g = ops.blockdiag_glu(a16, self.gated_layers.weight_bf16())
+            g = self.glu(a16)
             return ops.blockdiag_linear_layernorm(g, w, self.wo.bias.detach().float().contiguous(), a16, gamma, beta, eps,
                                                   want_f32=want_f32, want_bf16=want_bf16,
                                                   want_channel_major=want_channel_major)

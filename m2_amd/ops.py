@@ -272,6 +272,46 @@ def mlp_fused(x: Tensor, w_gated: Tensor, w_out: Tensor, bias: Optional[Tensor] 
     return out
 
 
+def glu_stream_supported(in_features: int, intermediate: int, nblocks: int) -> bool:
+    return bool(lib.m2_glu_stream_supported(int(in_features), int(intermediate), int(nblocks)))
+
+
+def glu_stream_pack(w_gated: Tensor) -> Tensor:
+    """gated_layers.weight (nb, 2I/nb, d/nb) bf16 -> the packed copy `glu_stream` streams (flat bf16 tensor of the
+    weight's size).  Once per set of weights."""
+    nb, q, p = w_gated.shape
+    _require(w_gated, "w_gated", torch.bfloat16)
+    d, I = nb * p, nb * q // 2
+    nbytes = int(lib.m2_glu_stream_packed_bytes(d, I, nb))
+    if nbytes == 0:
+        raise RuntimeError(f"glu_stream is built for nblocks=4, in_features=1536, intermediate % 128 == 0; got {nb}, {d}, {I}")
+    packed = torch.empty(nbytes // 2, dtype=torch.bfloat16, device=w_gated.device)
+    check(lib.m2_glu_stream_pack(_ptr(w_gated), _ptr(packed), d, I, nb, _stream()))
+    return packed
+
+
+def glu_stream(x: Tensor, w_gated: Tensor, out: Optional[Tensor] = None, packed: Optional[Tensor] = None) -> Tensor:
+    """gelu_erf(h[:, :I]) * h[:, I:] with h = blockdiag(x, w_gated), as `blockdiag_glu`, for 384-wide blocks.
+    x (M, d) bf16, w_gated (nb, 2I/nb, d/nb) bf16; `packed` = glu_stream_pack(w_gated), which a caller with fixed
+    weights computes once (without it the weight is packed on every call)."""
+    M, d = x.shape
+    nb, q, p = w_gated.shape
+    _require(x, "x", torch.bfloat16)
+    I = nb * q // 2
+    if nb * p != d:
+        raise ValueError(f"x has {d} features, w_gated expects {nb}*{p}")
+    if packed is None:
+        packed = glu_stream_pack(w_gated)
+    else:
+        _require(packed, "packed", torch.bfloat16, (int(lib.m2_glu_stream_packed_bytes(d, I, nb)) // 2,))
+    if out is None:
+        out = torch.empty(M, I, dtype=torch.bfloat16, device=x.device)
+    else:
+        _require(out, "out", torch.bfloat16, (M, I))
+    check(lib.m2_glu_stream_fwd(_ptr(x), _ptr(packed), _ptr(out), M, d, I, nb, _stream()))
+    return out
+
+
 def layernorm(x: Tensor, gamma: Tensor, beta: Tensor, eps: float, want_f32: bool = True, want_bf16: bool = False,
               want_channel_major: bool = False):
     """LayerNorm over the last dim of x (M, d) fp32 or bf16 -> (f32 (M,d) | None, bf16 (M,d) | None, f32 (d,M) | None)."""

@@ -695,3 +695,33 @@ def test_blockdiag_linear_fp32_outside_autocast(gpu, M, in_f, out_f, nb):
         assert low.dtype == torch.bfloat16
         e = rel_err(low.float(), ref)[0]
         assert 1e-4 < e < TOL_BF16, e
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,I", [(1, 6144), (100, 6144), (128, 6144), (300, 1536), (8192, 6144), (8192 - 70, 6144), (130, 256),
+                                 (520, 128)])
+def test_glu_stream_matches_oracle_and_the_tiled_kernel(gpu, M, I):
+    """gated_layers -> GLU for 384-wide blocks (d = 1536) from packed weights, against fp64 on the bf16-rounded
+    operands and against m2_blockdiag_glu_fwd (same arithmetic: bit-close, the accumulation order differs), ragged M,
+    one chunk per r (I = 128), more rows than one round of workgroups."""
+    from m2_amd import ops
+    from oracle import m2_oracle as O
+    d, nb = 1536, 4
+    assert ops.glu_stream_supported(d, I, nb) and not ops.glu_stream_supported(768, 3072, nb)
+    g = torch.Generator().manual_seed(7 * M + I)
+    x = torch.randn(M, d, generator=g).bfloat16()
+    wg = (torch.randn(nb, 2 * I // nb, d // nb, generator=g) * 0.05).bfloat16()
+    got = ops.glu_stream(x.to(gpu), wg.to(gpu))
+    h = O.blockdiag_multiply(x.float(), wg.float()).double()
+    ref = torch.nn.functional.gelu(h[:, :I]) * h[:, I:]
+    assert got.shape == (M, I) and got.dtype == torch.bfloat16
+    assert rel_err(got.float(), ref)[0] < TOL_BF16
+    tiled = ops.blockdiag_glu(x.to(gpu), wg.to(gpu))
+    assert rel_err(got.float(), tiled.float().double())[0] < 1e-2      # both rounded to bf16: an ulp apart at most
+    # the packed weight can be computed once and handed in
+    pk = ops.glu_stream_pack(wg.to(gpu))
+    again = ops.glu_stream(x.to(gpu), wg.to(gpu), packed=pk)
+    assert torch.equal(again, got)
+    with pytest.raises(RuntimeError, match="1536"):
+        ops.glu_stream(torch.zeros(8, 768, device=gpu, dtype=torch.bfloat16),
+                       torch.zeros(4, 256, 192, device=gpu, dtype=torch.bfloat16))
