@@ -152,92 +152,6 @@ def cpu_baseline(sd, cfg, ids, mask, B):
                            f"(min {times[0]:.2f}, max {times[2]:.2f})"}
 
 
-def probe_matrix_pipe(iters: int = 4000):
-    """Sustained bf16 MFMA rate of the chip (m2_probe_mfma_fwd) alone and with the company real kernels give it."""
-    import ctypes
-    from m2_amd._lib import check, lib
-    sink = torch.empty(512 * 1024, device="cuda:0")
-    rows = []
-    for reads, valu in ((0, 0), (1, 0), (2, 0), (1, 4), (1, 6), (1, 11)):
-        for wps in (1, 2):
-            n, waves = ctypes.c_longlong(0), ctypes.c_int(0)
-            call = lambda it: check(lib.m2_probe_mfma_fwd(reads, valu, wps, it, ctypes.c_void_p(sink.data_ptr()),
-                                                          ctypes.byref(n), ctypes.byref(waves),
-                                                          torch.cuda.current_stream().cuda_stream))
-            call(10)
-            torch.cuda.synchronize()
-            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s.record()
-            call(iters)
-            e.record()
-            torch.cuda.synchronize()
-            ms = s.elapsed_time(e)
-            tflops = n.value * waves.value * 32768 / (ms * 1e-3) / 1e12
-            rows.append({"lds_reads_per_mfma": reads, "valu_per_mfma": valu, "waves_per_simd": wps, "ms": ms,
-                         "tflops": tflops, "frac_of_published_peak": tflops / MFMA_BF16_PEAK_TFLOPS})
-    return {"probe": "v_mfma_f32_32x32x16_bf16 loop on all compute units", "published_peak_tflops": MFMA_BF16_PEAK_TFLOPS,
-            "rows": rows, "dft16_pass": probe_dft16_pass(), "l2_stream": probe_l2_stream()}
-
-
-def probe_l2_stream(iters: int = 2000):
-    """What one compute unit pulls out of L2 into LDS when all of them do (m2_probe_l2_stream_fwd)."""
-    import ctypes
-    from m2_amd._lib import check, lib
-    region = torch.ones(1 << 20, device="cuda:0", dtype=torch.float32)      # 4 MiB
-    sink = torch.zeros(512, device="cuda:0")
-    out = []
-    for mode, name in ((0, "direct-to-LDS loads, sixteen 64-byte row pieces per instruction"),
-                       (1, "direct-to-LDS loads, 1 KB contiguous per instruction"),
-                       (2, "plain 16-byte loads, software-pipelined, then LDS writes"),
-                       (3, "direct-to-LDS loads, eight whole 128-byte lines per instruction")):
-        wgs = ctypes.c_int(0)
-        call = lambda it: check(lib.m2_probe_l2_stream_fwd(mode, it, ctypes.c_void_p(region.data_ptr()), 1 << 20,
-                                                           ctypes.c_void_p(sink.data_ptr()), ctypes.byref(wgs),
-                                                           torch.cuda.current_stream().cuda_stream))
-        call(10)
-        torch.cuda.synchronize()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        call(iters)
-        e.record()
-        torch.cuda.synchronize()
-        us_per_iter = s.elapsed_time(e) * 1e3 / iters
-        out.append({"mode": name, "us_per_40KB": us_per_iter, "GBps_per_compute_unit": 40960 / us_per_iter / 1e3,
-                    "TBps_all": wgs.value * 40960 / us_per_iter / 1e6, "workgroups": wgs.value})
-    return out
-
-
-def probe_dft16_pass(nrows: int = 1024, iters: int = 200):
-    """The radix-16 pass of the L = 8192 half transform on the vector ALU against the same pass as a split-bf16 MFMA
-    product (m2_probe_dft16_pass_fwd): time per pass over `nrows` LDS-resident rows, and how far one MFMA pass is
-    from one vector-ALU pass on the same random rows."""
-    import ctypes
-    from m2_amd._lib import check, lib
-    stream = lambda: torch.cuda.current_stream().cuda_stream
-    x = torch.randn(nrows, 8192, 2, device="cuda:0", generator=torch.Generator(device="cuda:0").manual_seed(1))
-    out = {}
-    one = {}
-    for name, mode in (("valu", 0), ("mfma_split_bf16", 1)):
-        y = x.clone()
-        check(lib.m2_probe_dft16_pass_fwd(mode, 1, nrows, ctypes.c_void_p(y.data_ptr()), stream()))
-        one[name] = y
-        z = (x * 1e-3).clone()
-        check(lib.m2_probe_dft16_pass_fwd(mode, 2, nrows, ctypes.c_void_p(z.data_ptr()), stream()))
-        torch.cuda.synchronize()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        z = torch.zeros_like(x)                      # zeros stay zeros: no overflow over many unnormalised passes
-        s.record()
-        check(lib.m2_probe_dft16_pass_fwd(mode, iters, nrows, ctypes.c_void_p(z.data_ptr()), stream()))
-        e.record()
-        torch.cuda.synchronize()
-        out[name + "_us_per_pass"] = s.elapsed_time(e) * 1e3 / iters
-    ref = one["valu"].double()
-    out["mfma_vs_valu_max_rel"] = ((one["mfma_split_bf16"].double() - ref).abs().max() / ref.abs().max()).item()
-    out["mfma_vs_valu_l2_rel"] = ((one["mfma_split_bf16"].double() - ref).norm() / ref.norm()).item()
-    out["rows"], out["iters"] = nrows, iters
-    return out
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -254,36 +168,16 @@ def main():
                          "sit inside a graph, so the same K steps run eagerly first, with HIP events around "
                          "every launch, for the roofline object and eager_ms_per_step")
     ap.set_defaults(hip_graph=True)
-    ap.add_argument("--probe", action="store_true",
-                    help="only measure what the matrix pipe sustains on this chip (MFMA loop alone, with LDS operand "
-                         "reads, with vector-ALU work beside it) and exit")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="only run a plain 256 MiB device copy three times (known-size kernel for scaling "
-                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
 
-    if args.calibrate_copy:
-        n = 256 * 1024 * 1024 // 4
-        src = torch.zeros(n, device="cuda:0")
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"calibrate_copy_bytes_read": n * 4, "calibrate_copy_bytes_written": n * 4, "repeats": 3}))
-        return
-
     import __graft_entry__
     __graft_entry__.ensure_built()          # compiles only when the tree holds no library yet
     import m2_amd
     from m2_amd import ops
-
-    if args.probe:
-        print(json.dumps(probe_matrix_pipe()))
-        return
 
     cfg, B, L, ids, mask, label, idx = workload(args.config)
     d = cfg.hidden_size

@@ -248,34 +248,6 @@ int m2_embed_layernorm_fwd(const long long* input_ids, const long long* token_ty
                            float* out_f32, void* out_bf16, float* out_channel_major, int* bad_index, int B, int L,
                            int d, void* stream);
 
-/* ---------------------------------------------------------------------------------------------
- * Measurement aid (no counterpart in the reference): a loop of 12 * iters v_mfma_f32_32x32x16_bf16 per wave on every
- * compute unit, alone or accompanied by 1 or 2 software-pipelined 16-byte LDS operand reads per MFMA and by 0, 4, 6
- * or 11 fp32 FMAs per MFMA in the same wave, at 1 or 2 waves per SIMD.  The caller times the stream around the call;
- * 32768 flop per MFMA, *mfma_per_wave MFMAs in each of *waves waves.  bench.py --probe prints the rates: they are the
- * ceilings the GEMM-shaped kernels are held against beside the published peak.  sink: device buffer of at least
- * 512 floats per compute unit (written so that the loop is not optimised away).
- * Supported (lds_reads_per_mfma, valu_per_mfma): (0,0) (1,0) (2,0) (1,4) (1,6) (1,11). */
-int m2_probe_mfma_fwd(int lds_reads_per_mfma, int valu_per_mfma, int waves_per_simd, int iters, float* sink,
-                      long long* mfma_per_wave, int* waves, void* stream);
-
-/* Measurement aid (no counterpart in the reference): the radix-16 pass (stride 16, with its twiddles) of the L = 8192
- * half transform used by the long-convolution kernels, repeated `iters` times in place on nrows rows of 8192
- * complex64 points (rows: device pointer, nrows * 8192 * 2 floats), each row resident in the LDS of one workgroup.
- * use_mfma == 0: butterflies on the vector ALU (what m2_mixer_core_fwd runs); use_mfma != 0: the same pass as a
- * product with the real 32 x 32 form of the 16-point DFT matrix on bf16 MFMA, operands split into bf16 high / low
- * parts (three products).  bench.py --probe times the two against each other and reports their difference. */
-int m2_probe_dft16_pass_fwd(int use_mfma, int iters, int nrows, float* rows, void* stream);
-
-/* Measurement probe: the L2 -> LDS stream one compute unit sustains when all do.  One 512-thread workgroup per
- * compute unit copies the same `region` (>= 1 MiB of device memory, L2-resident after the first pass) into LDS,
- * 40 KB per iteration with a barrier, by direct-to-LDS loads that gather sixteen 64-byte row pieces per instruction
- * (mode 0), direct-to-LDS loads of 1 KB contiguous per instruction (mode 1), software-pipelined plain loads
- * followed by LDS writes (mode 2), or direct-to-LDS loads that gather eight whole 128-byte lines (mode 3).  `sink`: 512 floats; *workgroups receives the number of workgroups launched.
- * Bytes moved = workgroups * iters * 40960. */
-int m2_probe_l2_stream_fwd(int mode, int iters, const void* region, long region_bytes, float* sink, int* workgroups,
-                           void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -194,9 +194,21 @@ class BertGatedLinearUnitMLP(nn.Module):
                              want_channel_major=want_channel_major)
 
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        """fp32 input outside CUDA autocast runs in fp32 throughout, as the reference's modules do there
+        (bert/src/bert_layers.py:482-508 with bert/src/mm/blockdiag_multiply.py:50 casting only under autocast);
+        bf16 input or an enclosing autocast takes the bf16 kernels of the fused schedule."""
         if self.training and self.dropout.p > 0:
             raise NotImplementedError("m2_amd is a forward/inference path: call .eval() first")
         shape = hidden_states.shape
+        gamma, beta, eps = self.ln_params()
+        if hidden_states.dtype == torch.float32 and not torch.is_autocast_enabled():
+            x = hidden_states.reshape(-1, shape[-1]).contiguous()
+            h = self.gated_layers(x)                                   # fp32 block-diagonal kernel
+            I = self.config.intermediate_size
+            g = self.act(h[:, :I]) * h[:, I:]
+            s = self.wo(g.contiguous()) + x
+            o32, _, _ = ops.layernorm(s.contiguous(), gamma, beta, eps, want_f32=True)
+            return o32.view(shape)
         a16 = hidden_states.reshape(-1, shape[-1]).to(torch.bfloat16).contiguous()
         o32, _, _ = self.normed(a16, True, False, False)
         return o32.view(shape)
@@ -218,8 +230,10 @@ class BertLayer(nn.Module):
 
     def forward(self, hidden_states, cu_seqlens=None, seqlen=None, subset_idx=None, indices=None, attn_mask=None,
                 bias=None) -> torch.Tensor:
-        with torch.autocast("cuda", dtype=torch.bfloat16):
-            a, _ = self.attention(hidden_states)
+        # No autocast is forced here: like the reference's layer (bert/src/bert_layers.py:575-599) this runs in
+        # whatever precision the caller set up -- fp32 input outside autocast stays fp32 end to end, bf16 input or an
+        # enclosing torch.autocast("cuda", dtype=torch.bfloat16) takes the bf16 GEMM kernels.
+        a, _ = self.attention(hidden_states)
         return self.mlp(a)
 
     def fused(self, h16: Optional[torch.Tensor], hT: Optional[torch.Tensor], B: int, L: int, want_f32: bool,

@@ -54,6 +54,32 @@ def test_hyena_filter_taps(gpu, L, std):
         assert rel_err(hr.cpu(), kr.T[None])[0] < max(2e-5, 4 * e32)
 
 
+@pytest.mark.parametrize("L", [8192, 32768])
+def test_hyena_filter_taps_at_benchmark_lengths(gpu, L):
+    """Filter taps at the benchmark's own sizes (d = 768, L = 8192 and 32768: the 64-position hidden tiles and the
+    256-position projection runs) against the fp64 oracle, with the fp32 CPU oracle's own distance from fp64 as the
+    yardstick, both filters of a mixer, N(0, 0.02) weights as in the benchmark."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    cfg = m2_amd.m2_bert_80m(L)
+    sd = m2_amd.seeded_state_dict(cfg, 1234, what="mixer")
+    mix = m2_amd.MonarchMixerSequenceMixing(768, l_max=L, bidirectional=True, hyena_emb_dim=5, hyena_filter_order=128,
+                                            residual_long_conv=True, hyena_w=10)
+    mix.load_state_dict(sd)
+    mix = mix.to(gpu)
+    sd64 = O.cast_state_dict(sd, torch.float64)
+    for fn, name in ((mix.filter_fn, "filter_fn."), (mix.filter_fn2, "filter_fn2.")):
+        taps = fn.bidirectional_taps(L).cpu()
+        ref = O.bidirectional_kernel(O.hyena_filter_taps(sd64, name, L, rev=False)[0].T,
+                                     O.hyena_filter_taps(sd64, name, L, rev=True)[0].T, L)
+        ref32 = O.bidirectional_kernel(O.hyena_filter_taps(sd, name, L, rev=False)[0].T,
+                                       O.hyena_filter_taps(sd, name, L, rev=True)[0].T, L)
+        e32, _ = rel_err(ref32, ref)
+        e, e2 = rel_err(taps, ref)
+        print(f"taps L={L} {name}: max-rel {e:.2e} L2-rel {e2:.2e} (fp32 CPU oracle vs fp64: {e32:.2e})")
+        assert e < max(2e-5, 4 * e32), (name, e, e32)
+
+
 @pytest.mark.parametrize("L", [128, 256, 512, 1024, 2048, 4096, 8192, 16384, 32768])
 @pytest.mark.parametrize("act", ["f32", "bf16"])
 def test_mixer_core(gpu, L, act):
