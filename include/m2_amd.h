@@ -88,6 +88,26 @@ int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int 
 int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order,
                                int emb_dim, float w_mod, float shift, float* taps, void* stream);
 
+/* All implicit filters of a batch of mixers -> the spectra m2_mixer_core_fwd reads, in one call: the whole of
+ * HyenaFilter.filter / filter_rev (+ modulation), the bidirectional window, the skip weight and rfft(k) / 2L for
+ * every mixer of a model at once (bert/src/mm/monarch_mixer_sequence_mixer.py:120-139 with
+ * bert/src/mm/hyena_utils.py:201-236 and :24-33; the reference's native filter kernel is batched over filters the
+ * same way, csrc/flashmm/flash_mm.cpp:301-338).  Same arithmetic as m2_hyena_filter_fwd followed by
+ * m2_filter_spectrum_fwd per mixer, in three or four launches for ALL mixers; for L <= 512 the output projection,
+ * the decay and the transform are one kernel and the taps never exist in memory.
+ * params_dev  DEVICE array of nmixers * filters_per_mixer structs (of device pointers): filter_fn of mixer 0,
+ *             filter_fn2 of mixer 0 (when filters_per_mixer == 2), filter_fn of mixer 1, ...  All filters share L, d,
+ *             order, emb_dim; a filter is bidirectional when its rw0 .. rw3 are non-null.  The library cannot check
+ *             pointers that live in device memory: the caller guarantees the forward-MLP pointers are valid.
+ * skip_dev    DEVICE array of nmixers * filters_per_mixer pointers to the (d) fp32 skip weights (filter_fn.bias),
+ *             entries may be null; the array itself may be NULL (no skip weights).
+ * workspace   m2_mixer_filters_workspace_bytes(...) bytes of device memory, 256-byte aligned.
+ * spec        nmixers consecutive buffers of m2_filter_spectrum_bytes(d, L) bytes. */
+size_t m2_mixer_filters_workspace_bytes(int nmixers, int filters_per_mixer, int L, int d, int order);
+int m2_mixer_filters_fwd(const m2_hyena_filter_params* params_dev, const float* const* skip_dev, int nmixers,
+                         int filters_per_mixer, int L, int d, int order, int emb_dim, float w_mod, float shift,
+                         void* workspace, float* spec, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Long convolution: filter spectra and the fused mixer core.
  * Stand in for: bert/src/mm/hyena_utils.py:16-42 (fftconv_ref), :219-248 (HyenaFilter.forward) and

@@ -298,4 +298,37 @@ __device__ __forceinline__ void inverse_from_pairs(cf (&x)[16], int t, float2* r
   inv_load_compute<P, 1, P::R1, P::S1, LOWER_ONLY>(x, t, row, tw);
 }
 
+// After forward_to_pairs on z = k1 + i k2 (two real filters packed into one complex row): separates the two
+// spectra and stores them in the order the mixer core's multiply reads them, sp[slot * T] as float4 = (K1.re,
+// K1.im, K2.re, K2.im) for the frequency in slot `slot` of this work item's group; work item 0 holds DC and Nyquist
+// (real, packed into slot 0) and the two self-mirrored groups.  `scale` carries the 1/2 of the separation and the
+// 1/N of the convolution.
+template <class P>
+__device__ __forceinline__ void store_filter_spectrum(const cf (&x)[16], int t, float scale, float4* __restrict__ sp) {
+  float4 K[8];
+  auto split = [&](cf za, cf zb) -> float4 {
+    // K1 = (za + conj zb) * scale ; K2 = (za - conj zb) / i * scale
+    return make_float4(scale * (za.re + zb.re), scale * (za.im - zb.im), scale * (za.im + zb.im),
+                       scale * (zb.re - za.re));
+  };
+  if (t != 0) {
+    static_for<0, 8>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      K[j] = split(x[bitrev(j, 3)], x[8 + bitrev(7 - j, 3)]);
+    });
+  } else {
+    const cf z0 = x[bitrev(0, 3)], z4 = x[bitrev(4, 3)];
+    K[0] = make_float4(2.f * scale * z0.re, 2.f * scale * z4.re, 2.f * scale * z0.im, 2.f * scale * z4.im);
+    static_for<1, 4>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      K[j] = split(x[bitrev(j, 3)], x[bitrev(8 - j, 3)]);
+    });
+    static_for<0, 4>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      K[4 + j] = split(x[8 + bitrev(j, 3)], x[8 + bitrev(7 - j, 3)]);
+    });
+  }
+  static_for<0, 8>([&](auto s) { sp[decltype(s)::value * P::T] = K[decltype(s)::value]; });
+}
+
 }  // namespace m2

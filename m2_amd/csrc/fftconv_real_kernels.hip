@@ -36,6 +36,7 @@
 
 #include "fft_engine.h"
 #include "fft_split.h"
+#include "hyena_filter.h"
 #include "row_io.h"
 
 namespace m2 {
@@ -347,12 +348,17 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
 // ------------------------------------------------------------------------------------------
 template <class P>
 __global__ __launch_bounds__(P::T) void filter_spectrum_real_kernel(
-    const float* __restrict__ taps1,    // (d, 2 LS) bidirectional taps of filter_fn
-    const float* __restrict__ taps2,    // (d, 2 LS) bidirectional taps of filter_fn2 (null: its blocks are zeroed)
-    const float* __restrict__ D1,       // (d) skip weight of filter_fn, added to tap 0 (may be null)
-    const float* __restrict__ D2,       // (d) skip weight of filter_fn2 (may be null)
-    float* __restrict__ spec, int d) {
+    const float* taps1,    // (d, 2 LS) bidirectional taps of filter_fn
+    const float* taps2,    // (d, 2 LS) bidirectional taps of filter_fn2 (null: its blocks are zeroed)
+    const float* D1,       // (d) skip weight of filter_fn, added to tap 0 (may be null)
+    const float* D2,       // (d) skip weight of filter_fn2 (may be null)
+    float* __restrict__ spec, int d, SpectrumBatch sb) {
   constexpr int NS = P::L, H = P::N, T = P::T, R1 = P::R1, R2 = P::R2;
+  {
+    float* sp = spec;
+    select_mixer(sb, d, 2 * H, taps1, taps2, D1, D2, sp);
+    spec = sp;
+  }
   constexpr long BLK = real_spec_block<P>();
   extern __shared__ float2 lds[];
   float2* row = lds;
@@ -485,7 +491,7 @@ int launch_mixer_real_dispatch(const void* xproj, const float* u, const float* s
 }
 
 int launch_filter_spectrum_real(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
-                                int d, hipStream_t stream) {
+                                int d, const SpectrumBatch& sb, int nmixers, hipStream_t stream) {
   typedef RealPlan P;
   const size_t lds_bytes = (size_t)P::WG_LDS * sizeof(float2);
   auto kern = filter_spectrum_real_kernel<P>;
@@ -493,7 +499,7 @@ int launch_filter_spectrum_real(const float* taps1, const float* taps2, const fl
   if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(filter_spectrum_real): %s", hipGetErrorString(e));
   int grid = num_cus();
   if (grid > 2 * d) grid = 2 * d;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(P::T), lds_bytes, stream, taps1, taps2, D1, D2, spec, d);
+  hipLaunchKernelGGL(kern, dim3(grid, nmixers), dim3(P::T), lds_bytes, stream, taps1, taps2, D1, D2, spec, d, sb);
   return check_launch("filter_spectrum_real");
 }
 

@@ -30,6 +30,7 @@
 
 #include "fft_engine.h"
 #include "fft_split.h"
+#include "hyena_filter.h"
 #include "row_io.h"
 
 namespace m2 {
@@ -205,17 +206,22 @@ __global__ __launch_bounds__(P::T) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
 // ------------------------------------------------------------------------------------------
 template <class P, bool HAS2>
 __global__ __launch_bounds__(P::T) void filter_spectrum_split_kernel(
-    const float* __restrict__ taps1,    // (d, N) bidirectional taps of filter_fn
-    const float* __restrict__ taps2,    // (d, N) bidirectional taps of filter_fn2 (may be null)
-    const float* __restrict__ D1,       // (d) skip weight of filter_fn, added to tap 0 (may be null)
-    const float* __restrict__ D2,       // (d) skip weight of filter_fn2 (may be null)
+    const float* taps1,    // (d, N) bidirectional taps of filter_fn
+    const float* taps2,    // (d, N) bidirectional taps of filter_fn2 (may be null)
+    const float* D1,       // (d) skip weight of filter_fn, added to tap 0 (may be null)
+    const float* D2,       // (d) skip weight of filter_fn2 (may be null)
     float4* __restrict__ spec,          // (d, 2, 16, T)
-    int d) {
+    int d, SpectrumBatch sb) {
   constexpr int L = P::L, N = P::N, T = P::T;
   extern __shared__ float2 lds[];
   float2* row = lds;
   float2* tab2 = lds + P::ROW_LDS;
   const int t = threadIdx.x;
+  {
+    float* sp = reinterpret_cast<float*>(spec);
+    select_mixer(sb, d, N, taps1, taps2, D1, D2, sp);
+    spec = reinterpret_cast<float4*>(sp);
+  }
 
   tab2_init<P>(tab2);
   cf b[P::NB1];
@@ -339,9 +345,10 @@ static int launch_mixer_split(const void* xproj, const float* u, const float* sw
 
 template <class P>
 static int launch_filter_spectrum_split_t(const float* taps1, const float* taps2, const float* D1, const float* D2,
-                                          float* spec, int d, hipStream_t stream) {
+                                          float* spec, int d, const SpectrumBatch& sb, int nmixers, hipStream_t stream) {
   const size_t lds_bytes = (size_t)P::WG_LDS * sizeof(float2);
-  auto kern = taps2 ? filter_spectrum_split_kernel<P, true> : filter_spectrum_split_kernel<P, false>;
+  const bool has2 = sb.taps ? sb.fpm == 2 : taps2 != nullptr;
+  auto kern = has2 ? filter_spectrum_split_kernel<P, true> : filter_spectrum_split_kernel<P, false>;
   if (lds_bytes > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(filter_spectrum_split): %s", hipGetErrorString(e));
@@ -352,7 +359,7 @@ static int launch_filter_spectrum_split_t(const float* taps1, const float* taps2
   // a multiple of 16 workgroups: an even number per XCD, so that the two halves of a channel run side by side
   int grid = (num_cus() * per_cu) / 16 * 16;
   if (grid > 2 * d) grid = 2 * d;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(P::T), lds_bytes, stream, taps1, taps2, D1, D2, (float4*)spec, d);
+  hipLaunchKernelGGL(kern, dim3(grid, nmixers), dim3(P::T), lds_bytes, stream, taps1, taps2, D1, D2, (float4*)spec, d, sb);
   return check_launch("filter_spectrum_split");
 }
 
@@ -388,11 +395,11 @@ int launch_mixer_split_dispatch(const void* xproj, const float* u, const float* 
 }
 
 int launch_filter_spectrum_split(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
-                                 int d, int L, hipStream_t stream) {
+                                 int d, int L, const SpectrumBatch& sb, int nmixers, hipStream_t stream) {
   switch (L) {
 #define X(LOGL, R1, R2) \
   case 1 << LOGL:       \
-    return launch_filter_spectrum_split_t<SplitPlan<LOGL, R1, R2>>(taps1, taps2, D1, D2, spec, d, stream);
+    return launch_filter_spectrum_split_t<SplitPlan<LOGL, R1, R2>>(taps1, taps2, D1, D2, spec, d, sb, nmixers, stream);
     M2_FOR_EACH_SPLIT_PLAN(X)
 #undef X
   }

@@ -20,30 +20,11 @@
 
 #include <mutex>
 
-#include "fft_regs.h"
-#include "m2_internal.h"
+#include "hyena_filter.h"
 
 namespace m2 {
 
-constexpr int kOrder = 128;
-constexpr int kMaxEmb = 8;
 constexpr int kPosTile = 32;      // positions per workgroup in hidden_kernel
-
-struct MlpPtrs {
-  const float *w0, *b0, *w1, *b1, *w2, *b2, *w3;
-};
-struct FilterPtrs {
-  const float *z, *t, *freq, *deltas;
-  MlpPtrs mlp[2];                 // [0] forward, [1] reverse
-};
-constexpr int kMaxFilters = 4;
-struct FilterBatch {
-  FilterPtrs f[kMaxFilters];
-};
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // sin(x) by two-constant Cody-Waite reduction to [-pi/2, pi/2] (fused multiply-adds keep the reduction
 // exact to ~1e-15 n) and the odd Taylor polynomial to x^11 (truncation 5.6e-8 at pi/2).  Absolute error
@@ -68,28 +49,21 @@ __device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, 
   return __builtin_bit_cast(bf16x8, v);
 }
 
-// x = hi + mid + lo with three bf16 terms: 24 mantissa bits, i.e. all of an fp32 value
-__device__ __forceinline__ void split3(float x, float& hi, float& mid, float& lo) {
-  hi = bf16_to_f32(f32_to_bf16(x));
-  const float r = x - hi;
-  mid = bf16_to_f32(f32_to_bf16(r));
-  lo = r - mid;                      // the conversion of lo to bf16 happens where it is packed
-}
-
 // The 128 x 128 weights of the two inner layers, split into three bf16 parts and laid out as MFMA A operands, so
 // that hidden_kernel fetches them with coalesced 16-byte loads and no arithmetic:
 // wsplit[mlp][layer][part][wave w][K step ks][lane (i, h)] = 8 bf16 of row 32 w + i, K = 16 ks + 8 h .. + 7.
 // The d x 128 output projection likewise, in two parts (hi, lo), for project_kernel:
 // w3split[mlp][part][32-channel tile][K step ks][lane (i, h)] = 8 bf16 of row 32 tile + i, K = 16 ks + 8 h .. + 7.
 constexpr int kSplitPerLayer = 3 * kOrder * kOrder;      // bf16 elements per (mlp, layer)
-__global__ __launch_bounds__(256) void split_weights_kernel(FilterBatch fb, int nmlp, int d, uint16_t* __restrict__ wsplit,
+template <class TAB>
+__global__ __launch_bounds__(256) void split_weights_kernel(TAB tab, int nmlp, int d, uint16_t* __restrict__ wsplit,
                                                             uint16_t* __restrict__ w3split) {
   const int inner_blocks = nmlp * 2 * 4 * 8 * 64 / 256;
   if ((int)blockIdx.x >= inner_blocks) {
     const int id = ((int)blockIdx.x - inner_blocks) * 256 + threadIdx.x;      // (mlp, channel tile, ks, lane)
     const int lane = id & 63, ks = (id >> 6) & 7, ct = (id >> 9) % (d / 32), m = (id >> 9) / (d / 32);
     if (m >= nmlp) return;
-    const MlpPtrs& W = fb.f[m >> 1].mlp[m & 1];
+    const MlpPtrs& W = tab.at(m >> 1).mlp[m & 1];
     if (W.w3 == nullptr) return;
     const float* src = W.w3 + (long)(32 * ct + (lane & 31)) * kOrder + 16 * ks + 8 * (lane >> 5);
     float h[8], l[8];
@@ -108,7 +82,7 @@ __global__ __launch_bounds__(256) void split_weights_kernel(FilterBatch fb, int 
   const int id = blockIdx.x * 256 + threadIdx.x;             // (mlp, layer, wave, ks, lane)
   const int lane = id & 63, ks = (id >> 6) & 7, w = (id >> 9) & 3, layer = (id >> 11) & 1, m = id >> 12;
   if (m >= nmlp) return;
-  const MlpPtrs& W = fb.f[m >> 1].mlp[m & 1];
+  const MlpPtrs& W = tab.at(m >> 1).mlp[m & 1];
   if (W.w0 == nullptr) return;
   const float* src = (layer == 0 ? W.w1 : W.w2) + (long)(32 * w + (lane & 31)) * kOrder + 16 * ks + 8 * (lane >> 5);
   float h[8], md[8], l[8];
@@ -133,8 +107,8 @@ constexpr int kActRowB = 2 * kOrder + 16;     // bytes per padded bf16 row of an
 // weights pre-split by split_weights_kernel and held in registers for all tiles (fetching them is what a short run
 // of positions per workgroup pays most for: 96 KB per workgroup and layer from L2).  Within a layer the products of
 // tile i + 1 are issued together with the sin epilogue of tile i, so that matrix pipe and vector ALU overlap.
-template <int TILES>
-__global__ __launch_bounds__(256) void hidden_kernel(FilterBatch fb, int L, int emb, float w_mod,
+template <int TILES, class TAB>
+__global__ __launch_bounds__(256) void hidden_kernel(TAB tab, int L, int emb, float w_mod,
                                                      const uint16_t* __restrict__ wsplit,
                                                      uint16_t* __restrict__ h_hi /* (2 nf, L, 128) bf16 */,
                                                      uint16_t* __restrict__ h_lo /* (2 nf, L, 128) bf16 */) {
@@ -143,7 +117,7 @@ __global__ __launch_bounds__(256) void hidden_kernel(FilterBatch fb, int L, int 
   __shared__ float zt[P * kMaxEmb];
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
   const int fi = blockIdx.y >> 1, dir = blockIdx.y & 1;
-  const FilterPtrs& F = fb.f[fi];
+  const FilterPtrs& F = tab.at(fi);
   const MlpPtrs& W = F.mlp[dir];
   if (W.w0 == nullptr) return;                  // not bidirectional: nothing to do for dir == 1
   const int l0 = blockIdx.x * P;
@@ -287,13 +261,14 @@ __global__ __launch_bounds__(256) void hidden_kernel(FilterBatch fb, int L, int 
 // grid (L / kPosPerWg rounded up, d / 128 rounded up, 2 * nfilters).
 constexpr int kPosPerWg = 256;      // at most; 32-position tiles past L are skipped
 constexpr int kHRow = 2 * kOrder + 16;   // bytes per padded LDS row of one h3 part
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) void project_kernel(FilterBatch fb, int L, int d, float shift,
+template <class TAB>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) void project_kernel(TAB tab, int L, int d, float shift,
                                                       const uint16_t* __restrict__ h_hi, const uint16_t* __restrict__ h_lo,
                                                       const uint16_t* __restrict__ w3split,
                                                       float* __restrict__ taps /* (nf, d, 2L) */) {
   __shared__ __attribute__((aligned(16))) unsigned char hbuf[2][2][32 * kHRow];     // [buffer][hi, lo][row]
   const int fi = blockIdx.z >> 1, dir = blockIdx.z & 1;
-  const FilterPtrs& F = fb.f[fi];
+  const FilterPtrs& F = tab.at(fi);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i32 = lane & 31, half = lane >> 5;
   const int c0 = blockIdx.y * 128 + wave * 32;
   const bool active = c0 < d;                      // d is a multiple of 64: a wave is all in or all out
@@ -402,19 +377,51 @@ extern "C" size_t m2_hyena_filter_workspace_bytes(int nfilters, int L, int d, in
          (size_t)2 * nfilters * 2 * d * order * sizeof(uint16_t);
 }
 
-// Shared by the two entry points: validation and the two launches, `workspace` holding the h3 hi / lo parts.
-static int hyena_filter_launch(const char* who, const m2_hyena_filter_params* params, int nfilters, int L, int d,
-                               int order, int emb_dim, float w_mod, float shift, void* workspace, float* taps,
-                               void* stream) {
-  if (nfilters < 1 || nfilters > kMaxFilters)
-    return set_error(M2_ERR_UNSUPPORTED, "%s: nfilters=%d not in [1, %d]", who, nfilters, kMaxFilters);
+// The three launches of a batch of filters (weight re-split, hidden layers, projection + decay), the table coming
+// either by value or from device memory.  `w3split` / `taps` null: the projection is left to the caller (the fused
+// projection + spectrum kernel of short sequences, which splits the projection weights itself).
+template <class TAB>
+static int filter_launches(TAB tab, int nfilters, int L, int d, int emb_dim, float w_mod, float shift, uint16_t* h_hi,
+                           uint16_t* h_lo, uint16_t* wsplit, uint16_t* w3split, float* taps, hipStream_t s) {
+  const int inner_blocks = 2 * nfilters * 2 * 4 * 8 * 64 / 256;
+  const int split_blocks = inner_blocks + (w3split ? 2 * nfilters * (d / 32) * 8 * 64 / 256 : 0);
+  hipLaunchKernelGGL(split_weights_kernel<TAB>, dim3(split_blocks), dim3(256), 0, s, tab, 2 * nfilters, d, wsplit, w3split);
+  int rc = check_launch("hyena split_weights_kernel");
+  if (rc) return rc;
+  // positions per workgroup: longer runs amortise the weight fetch (96 KB per workgroup and layer), short sequences
+  // need the workgroups spread over the chip
+  if (L % 64 == 0 && L >= 1024)      // measured at L = 8192: 26.9 us with two tiles, 29.5 with four, 32.7 with one
+    hipLaunchKernelGGL((hidden_kernel<2, TAB>), dim3(L / 64, 2 * nfilters), dim3(256), 0, s, tab, L, emb_dim, w_mod, wsplit, h_hi, h_lo);
+  else
+    hipLaunchKernelGGL((hidden_kernel<1, TAB>), dim3(L / 32, 2 * nfilters), dim3(256), 0, s, tab, L, emb_dim, w_mod, wsplit, h_hi, h_lo);
+  rc = check_launch("hyena hidden_kernel");
+  if (rc || !taps) return rc;
+  hipLaunchKernelGGL(project_kernel<TAB>, dim3((L + kPosPerWg - 1) / kPosPerWg, (d + 127) / 128, 2 * nfilters), dim3(256), 0, s, tab, L, d, shift,
+                     h_hi, h_lo, w3split, taps);
+  return check_launch("hyena project_kernel");
+}
+
+static int check_filter_sizes(const char* who, int L, int d, int order, int emb_dim) {
   if (order != kOrder) return set_error(M2_ERR_UNSUPPORTED, "%s: order=%d, only 128 is built", who, order);
   if (emb_dim < 3 || emb_dim > kMaxEmb)
     return set_error(M2_ERR_UNSUPPORTED, "%s: emb_dim=%d not in [3, %d]", who, emb_dim, kMaxEmb);
   if (L <= 0 || L % kPosTile != 0)
     return set_error(M2_ERR_UNSUPPORTED, "%s: L=%d must be a positive multiple of %d", who, L, kPosTile);
   if (d <= 0 || d % 64 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: d=%d must be a positive multiple of 64", who, d);
-  FilterBatch fb;
+  return M2_OK;
+}
+
+// Shared by the two entry points that take a host array of filters: validation and the launches, `workspace`
+// holding the h3 hi / lo parts and the re-split weights.
+static int hyena_filter_launch(const char* who, const m2_hyena_filter_params* params, int nfilters, int L, int d,
+                               int order, int emb_dim, float w_mod, float shift, void* workspace, float* taps,
+                               void* stream) {
+  if (nfilters < 1 || nfilters > kMaxFilters)
+    return set_error(M2_ERR_UNSUPPORTED, "%s: nfilters=%d not in [1, %d]", who, nfilters, kMaxFilters);
+  int rc = check_filter_sizes(who, L, d, order, emb_dim);
+  if (rc) return rc;
+  TabByValue tab;
+  FilterBatch& fb = tab.fb;
   for (int f = 0; f < kMaxFilters; ++f) {
     const m2_hyena_filter_params& p = params[f < nfilters ? f : 0];
     if (!p.z || !p.t || !p.freq || !p.deltas || !p.w0 || !p.b0 || !p.w1 || !p.b1 || !p.w2 || !p.b2 || !p.w3)
@@ -427,26 +434,11 @@ static int hyena_filter_launch(const char* who, const m2_hyena_filter_params* pa
     fb.f[f].mlp[1] = rev ? MlpPtrs{p.rw0, p.rb0, p.rw1, p.rb1, p.rw2, p.rb2, p.rw3}
                          : MlpPtrs{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
   }
-  hipStream_t s = (hipStream_t)stream;
   uint16_t* h_hi = reinterpret_cast<uint16_t*>(workspace);
   uint16_t* h_lo = h_hi + (size_t)2 * nfilters * L * order;
   uint16_t* wsplit = h_lo + (size_t)2 * nfilters * L * order;
   uint16_t* w3split = wsplit + (size_t)2 * nfilters * 2 * 3 * order * order;
-  const int split_blocks = 2 * nfilters * 2 * 4 * 8 * 64 / 256 + 2 * nfilters * (d / 32) * 8 * 64 / 256;
-  hipLaunchKernelGGL(split_weights_kernel, dim3(split_blocks), dim3(256), 0, s, fb, 2 * nfilters, d, wsplit, w3split);
-  int rc = check_launch("hyena split_weights_kernel");
-  if (rc) return rc;
-  // positions per workgroup: longer runs amortise the weight fetch (96 KB per workgroup and layer), short sequences
-  // need the workgroups spread over the chip
-  if (L % 64 == 0 && L >= 1024)      // measured at L = 8192: 26.9 us with two tiles, 29.5 with four, 32.7 with one
-    hipLaunchKernelGGL(hidden_kernel<2>, dim3(L / 64, 2 * nfilters), dim3(256), 0, s, fb, L, emb_dim, w_mod, wsplit, h_hi, h_lo);
-  else
-    hipLaunchKernelGGL(hidden_kernel<1>, dim3(L / 32, 2 * nfilters), dim3(256), 0, s, fb, L, emb_dim, w_mod, wsplit, h_hi, h_lo);
-  rc = check_launch("hyena hidden_kernel");
-  if (rc) return rc;
-  hipLaunchKernelGGL(project_kernel, dim3((L + kPosPerWg - 1) / kPosPerWg, (d + 127) / 128, 2 * nfilters), dim3(256), 0, s, fb, L, d, shift,
-                     h_hi, h_lo, w3split, taps);
-  return check_launch("hyena project_kernel");
+  return filter_launches(tab, nfilters, L, d, emb_dim, w_mod, shift, h_hi, h_lo, wsplit, w3split, taps, (hipStream_t)stream);
 }
 
 extern "C" int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order,
@@ -510,4 +502,62 @@ extern "C" int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, 
   // left by an earlier (possibly longer) call is ever read and nothing needs clearing
   return hyena_filter_launch("m2_hyena_filter_fwd_static", params, nfilters, L, d, order, emb_dim, w_mod, shift, ptr,
                              taps, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// All filters of a batch of mixers -> their spectra, the pointer table in device memory.
+// ---------------------------------------------------------------------------------------------
+namespace {
+struct BatchLayout {
+  size_t h_lo, wsplit, w3split, taps, total;      // byte offsets into the workspace (h_hi at 0)
+  bool fused;                                     // projection + spectrum as one kernel, taps never in memory
+};
+BatchLayout batch_layout(int nmixers, int fpm, int L, int d) {
+  const size_t nf = (size_t)nmixers * fpm;
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  BatchLayout b;
+  b.fused = project_spectrum_supported(L);
+  b.h_lo = up(2 * nf * L * kOrder * sizeof(uint16_t));
+  b.wsplit = b.h_lo + up(2 * nf * L * kOrder * sizeof(uint16_t));
+  b.w3split = b.wsplit + up(2 * nf * 2 * 3 * kOrder * kOrder * sizeof(uint16_t));
+  b.taps = b.w3split + (b.fused ? 0 : up(2 * nf * 2 * (size_t)d * kOrder * sizeof(uint16_t)));
+  b.total = b.taps + (b.fused ? 0 : up(nf * (size_t)d * 2 * L * sizeof(float)));
+  return b;
+}
+}  // namespace
+
+extern "C" size_t m2_mixer_filters_workspace_bytes(int nmixers, int filters_per_mixer, int L, int d, int order) {
+  if (nmixers <= 0 || filters_per_mixer < 1 || filters_per_mixer > 2 || L <= 0 || d <= 0 || order != kOrder) return 0;
+  return batch_layout(nmixers, filters_per_mixer, L, d).total;
+}
+
+extern "C" int m2_mixer_filters_fwd(const m2_hyena_filter_params* params_dev, const float* const* skip_dev, int nmixers,
+                                    int filters_per_mixer, int L, int d, int order, int emb_dim, float w_mod,
+                                    float shift, void* workspace, float* spec, void* stream) {
+  const char* who = "m2_mixer_filters_fwd";
+  if (!params_dev || !workspace || !spec) return set_error(M2_ERR_ARG, "%s: null pointer", who);
+  if (nmixers < 1 || nmixers > 16384) return set_error(M2_ERR_ARG, "%s: nmixers=%d not in [1, 16384]", who, nmixers);
+  if (filters_per_mixer < 1 || filters_per_mixer > 2)
+    return set_error(M2_ERR_ARG, "%s: filters_per_mixer=%d must be 1 or 2", who, filters_per_mixer);
+  int rc = check_filter_sizes(who, L, d, order, emb_dim);
+  if (rc) return rc;
+  if (!m2_fftconv_supported_seqlen(L))
+    return set_error(M2_ERR_UNSUPPORTED, "%s: L=%d unsupported (need L a power of two in [128, 32768])", who, L);
+  const int nf = nmixers * filters_per_mixer;
+  const BatchLayout lay = batch_layout(nmixers, filters_per_mixer, L, d);
+  unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
+  uint16_t* h_hi = reinterpret_cast<uint16_t*>(ws);
+  uint16_t* h_lo = reinterpret_cast<uint16_t*>(ws + lay.h_lo);
+  uint16_t* wsplit = reinterpret_cast<uint16_t*>(ws + lay.wsplit);
+  uint16_t* w3split = lay.fused ? nullptr : reinterpret_cast<uint16_t*>(ws + lay.w3split);
+  float* taps = lay.fused ? nullptr : reinterpret_cast<float*>(ws + lay.taps);
+  TabByPointer tab{reinterpret_cast<const FilterPtrs*>(params_dev)};
+  hipStream_t s = (hipStream_t)stream;
+  rc = filter_launches(tab, nf, L, d, emb_dim, w_mod, shift, h_hi, h_lo, wsplit, w3split, taps, s);
+  if (rc) return rc;
+  const long spec_stride = (long)(m2_filter_spectrum_bytes(d, L) / sizeof(float));
+  if (lay.fused)
+    return launch_project_spectrum(tab.p, skip_dev, nmixers, filters_per_mixer, L, d, shift, h_hi, h_lo, spec, spec_stride, s);
+  SpectrumBatch sb{taps, skip_dev, filters_per_mixer, spec_stride};
+  return launch_filter_spectrum_any(nullptr, nullptr, nullptr, nullptr, spec, d, L, sb, nmixers, s);
 }

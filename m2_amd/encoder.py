@@ -277,6 +277,9 @@ class BertEncoder(nn.Module):
     Nothing in the captured region uses a memset."""
 
     UPFRONT_MAX_BYTES = 16 << 30
+    # device memory one batched filter-generation call may use for its workspace (hidden activations; for L > 512
+    # also the taps, 8 d L bytes per filter): the layers are generated in as few calls as stay below it
+    FILTER_WORKSPACE_BYTES = 2 << 30
 
     def __init__(self, config: M2BertConfig, use_hip_graph: bool = False):
         super().__init__()
@@ -285,17 +288,22 @@ class BertEncoder(nn.Module):
         self.num_attention_heads = config.num_attention_heads
         self.use_hip_graph = use_hip_graph
         self._graphs = {}
-        # Filter generation depends on the weights only, so it can run on a second stream (default priority):
-        #   "upfront"  all layers' spectra one after the other from the start of the forward, each layer waiting
-        #              for its own (holds all spectra at once: 100 MB per layer at L = 8192, d = 768);
+        # Filter generation depends on the weights only.
+        # batch_filters = True (default): the filters of ALL layers are generated at the start of the forward by
+        #   one library call per group of layers (m2_mixer_filters_fwd: a few launches for all of them; groups are
+        #   as large as FILTER_WORKSPACE_BYTES allows) -- on a second stream (default priority) beside the layers
+        #   unless overlap_filters is False, each layer waiting for its group.  Holds all spectra at once (16 d L
+        #   bytes per layer: 100 MB at L = 8192, d = 768) and is used while they stay below UPFRONT_MAX_BYTES.
+        # batch_filters = False, or spectra beyond UPFRONT_MAX_BYTES, or a layer with cache_filters: per layer, with
+        #   overlap_filters =
+        #   "upfront"  all layers' spectra one after the other on the second stream from the start of the forward;
         #   True       the spectra of layer i + 1 behind the mixer core of layer i;
         #   False      in line, on the main stream;
         #   None       "upfront" while all layers' spectra together stay below UPFRONT_MAX_BYTES, else True.
-        # Measured on MI355X, forward as one HIP graph, in line / "upfront" / True: 8.71 / 8.45 / 8.64 ms at
-        # L = 8192, B = 4; 15.22 / 14.54 / 14.89 ms at L = 32768, B = 1; 11.00 / 10.47 / 10.75 ms for 24 x 1536 at
-        # L = 128, B = 64.  Kernels of the two streams then share the chip, so per-kernel timings are taken in line.
+        self.batch_filters = True
         self.overlap_filters = None
         self._filter_stream = None
+        self._filter_table = None
         # nn.Module.load_state_dict of a parent never calls a child's load_state_dict, but it does run the
         # post hooks of every module it recursed into: new weights drop the captured graphs
         self.register_load_state_dict_post_hook(BertEncoder._drop_graphs_after_load)
@@ -335,7 +343,32 @@ class BertEncoder(nn.Module):
                 total = len(self.layer) * ops.lib.m2_filter_spectrum_bytes(d, L)
                 overlap = "upfront" if total <= self.UPFRONT_MAX_BYTES else True
             nxt = [None, None]                       # spectra of the next layer and the event that says they are ready
-            if overlap:
+            ahead = []
+            upfront = False
+            batched = self._batched_filter_plan(L)
+            if batched is not None:
+                # all layers' filters by a few launches per group of layers, beside the layers or ahead of them
+                table, groups = batched
+                f0 = self.layer[0].attention.filter_fn
+                side = None
+                if overlap is not False:
+                    if self._filter_stream is None:
+                        self._filter_stream = torch.cuda.Stream()          # default priority
+                    side = self._filter_stream
+                    side.wait_stream(cur)
+                with torch.cuda.stream(side if side is not None else cur):
+                    for first, count in groups:
+                        sp = ops.mixer_filter_spectra(table, w_mod=float(f0.w_mod), shift=float(f0.modulation.shift),
+                                                      first=first, count=count)
+                        ev = None
+                        if side is not None:
+                            sp.record_stream(cur)
+                            ev = torch.cuda.Event()
+                            ev.record(side)
+                        ahead += [(sp[j], ev) for j in range(count)]
+                upfront = True
+                overlap = "upfront" if side is not None else "inline-batched"
+            elif overlap:
                 if self._filter_stream is None:
                     self._filter_stream = torch.cuda.Stream()          # default priority
                 side = self._filter_stream
@@ -353,7 +386,6 @@ class BertEncoder(nn.Module):
                     nxt[0], nxt[1] = sp, ev
 
                 upfront = overlap == "upfront"
-                ahead = []
                 if upfront:          # all layers' spectra at once, in order, while the main stream runs the layers
                     side.wait_stream(cur)
                     with torch.cuda.stream(side):
@@ -382,9 +414,38 @@ class BertEncoder(nn.Module):
                                            after_core=hook, h32=o32)
                 if want:
                     outs.append(o32)
-            if overlap:
+            if overlap and overlap != "inline-batched":
                 cur.wait_stream(self._filter_stream)
         return outs
+
+    def _batched_filter_plan(self, L: int):
+        """(pointer table of all layers' filters, [(first layer, count), ...]) when the filters of all layers are
+        generated by batched calls, else None."""
+        if not self.batch_filters:
+            return None
+        mixers = [lay.attention for lay in self.layer]
+        m0 = mixers[0]
+        if any(m.cache_filters for m in mixers):
+            return None
+        same = all(m.d_model == m0.d_model and m.residual_long_conv == m0.residual_long_conv
+                   and m.bidirectional == m0.bidirectional and m.filter_fn.order == m0.filter_fn.order
+                   and m.filter_fn.emb_dim == m0.filter_fn.emb_dim and m.filter_fn.w_mod == m0.filter_fn.w_mod
+                   and m.filter_fn.modulation.shift == m0.filter_fn.modulation.shift for m in mixers)
+        d, n = m0.d_model, len(mixers)
+        if not same or n * ops.lib.m2_filter_spectrum_bytes(d, L) > self.UPFRONT_MAX_BYTES:
+            return None
+        entries = [m.filter_table_entry() for m in mixers]
+        probe = (L,) + tuple(t.data_ptr() for filters, skips in entries for f in filters for v in f.values()
+                             for t in (v if isinstance(v, list) else [v])) + tuple(b.data_ptr() for _, skips in entries
+                                                                                   for b in skips)
+        if self._filter_table is None or self._filter_table[0] != probe:
+            self._filter_table = (probe, ops.FilterTable([e[0] for e in entries], [e[1] for e in entries], L, d,
+                                                         m0.filter_fn.order, m0.filter_fn.emb_dim))
+        table = self._filter_table[1]
+        fpm = table.fpm
+        per = max(1, ops.lib.m2_mixer_filters_workspace_bytes(1, fpm, L, d, table.order))
+        group = max(1, min(n, self.FILTER_WORKSPACE_BYTES // per))
+        return table, [(i, min(group, n - i)) for i in range(0, n, group)]
 
     def _run_graphed(self, h32: Optional[torch.Tensor], B: int, L: int, all_layers: bool,
                      h16: Optional[torch.Tensor] = None, hT: Optional[torch.Tensor] = None) -> List[torch.Tensor]:

@@ -129,7 +129,10 @@ class HyenaFilter(OptimModule):
             p["fwd"] = self._mlp_tensors(self.implicit_filter)
             if which == "both" and self.bidirectional:
                 p["rev"] = self._mlp_tensors(self.implicit_filter_rev)
-        return {k: ([t.detach().float() for t in v] if isinstance(v, list) else v.detach().float()) for k, v in p.items()}
+        def plain(t):      # the kernels read fp32, contiguous tensors; parameters normally are, and then this is a view
+            t = t.detach()
+            return t if (t.dtype == torch.float32 and t.is_contiguous()) else t.float().contiguous()
+        return {k: ([plain(t) for t in v] if isinstance(v, list) else plain(v)) for k, v in p.items()}
 
     def _taps(self, L: int, which: str) -> torch.Tensor:
         if L > self.seq_len:

@@ -64,6 +64,7 @@ class MonarchMixerSequenceMixing(nn.Module):
         self.own_in_linear = False
         self.cache_filters = False
         self._spec_cache = None
+        self._filter_table = None
 
     # -- helpers -----------------------------------------------------------------------------
     def _cast(self, name: str, p: torch.Tensor, dtype) -> torch.Tensor:
@@ -95,13 +96,28 @@ class MonarchMixerSequenceMixing(nn.Module):
             return spec
         return self._generate_spectrum(L, fns)
 
+    def filter_table_entry(self):
+        """(filters, skip weights) of this mixer for an `ops.FilterTable`: filter_fn, then filter_fn2 if present."""
+        fns = [self.filter_fn] + ([self.filter_fn2] if self.residual_long_conv else [])
+        filters = [f.kernel_params("both") for f in fns]
+        skips = []
+        for f in fns:
+            b = f.bias.detach()
+            skips.append(b if (b.dtype == torch.float32 and b.is_contiguous()) else b.float().contiguous())
+        return filters, skips
+
     def _generate_spectrum(self, L: int, fns) -> torch.Tensor:
+        """All of filter generation in one library call: hidden layers, projection + decay, window, skip weight,
+        transform (for L <= 512 the taps never reach memory)."""
         f0 = self.filter_fn
-        taps = ops.hyena_filter_taps([f.kernel_params("both") for f in fns], L, self.d_model, f0.order, f0.emb_dim,
-                                     w_mod=float(f0.w_mod), shift=float(f0.modulation.shift))
-        D1 = self.filter_fn.bias.detach().float().contiguous()
-        D2 = self.filter_fn2.bias.detach().float().contiguous() if self.residual_long_conv else None
-        return ops.filter_spectrum(taps[0], taps[1] if self.residual_long_conv else None, D1, D2)
+        filters, skips = self.filter_table_entry()
+        table = self._filter_table
+        key_probe = (L,) + tuple(t.data_ptr() for f in filters for v in f.values()
+                                 for t in (v if isinstance(v, list) else [v])) + tuple(b.data_ptr() for b in skips)
+        if table is None or table[0] != key_probe:
+            table = (key_probe, ops.FilterTable([filters], [skips], L, self.d_model, f0.order, f0.emb_dim))
+            self._filter_table = table
+        return ops.mixer_filter_spectra(table[1], w_mod=float(f0.w_mod), shift=float(f0.modulation.shift))[0]
 
     def core(self, xproj: torch.Tensor, u_cm: Optional[torch.Tensor], B: int, L: int,
              spec: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -105,6 +105,83 @@ def hyena_filter_taps(filters: Sequence[dict], L: int, d: int, order: int, emb_d
     return taps
 
 
+class FilterTable:
+    """Pointer table, in device memory, of the implicit filters of a batch of mixers (what `m2_mixer_filters_fwd`
+    reads), with the tensors it points to kept alive.  Built once per set of parameter tensors (`key` = their
+    addresses): building it copies from the host, so it must happen outside a stream capture."""
+
+    def __init__(self, mixers: Sequence[Sequence[dict]], skips: Sequence[Sequence[Optional[Tensor]]], L: int, d: int,
+                 order: int, emb_dim: int):
+        self.nmixers = len(mixers)
+        self.fpm = len(mixers[0])
+        if self.fpm not in (1, 2) or any(len(m) != self.fpm for m in mixers) or any(len(k) != self.fpm for k in skips):
+            raise ValueError("every mixer must bring the same number (1 or 2) of filters and skip weights")
+        self.L, self.d, self.order, self.emb_dim = L, d, order, emb_dim
+        shapes = [(order, emb_dim), (order,), (order, order), (order,), (order, order), (order,), (d, order)]
+        rows, skip_row, keep = [], [], []
+        for filters, sk in zip(mixers, skips):
+            for f, D in zip(filters, sk):
+                z = f["z"].reshape(-1, emb_dim)[:L]
+                t = f["t"].reshape(-1)[:L]
+                freq = f["freq"].reshape(-1)
+                deltas = f["deltas"].reshape(-1)
+                _require(z, "z", torch.float32, (L, emb_dim))
+                _require(t, "t", torch.float32, (L,))
+                _require(freq, "freq", torch.float32, (order,))
+                _require(deltas, "deltas", torch.float32, (d,))
+                row = [z.data_ptr(), t.data_ptr(), freq.data_ptr(), deltas.data_ptr()]
+                keep += [z, t, freq, deltas]
+                for key in ("fwd", "rev"):
+                    ws = f.get(key)
+                    if ws is None:
+                        if key == "fwd":
+                            raise ValueError("filter without forward MLP")
+                        row += [0] * 7
+                        continue
+                    for w, s_ in zip(ws, shapes):
+                        _require(w, f"{key} MLP tensor", torch.float32, s_)
+                        keep.append(w)
+                        row.append(w.data_ptr())
+                rows.append(row)
+                if D is not None:
+                    _require(D, "skip weight", torch.float32, (d,))
+                    keep.append(D)
+                skip_row.append(0 if D is None else D.data_ptr())
+        self.keep = keep
+        self.key = (L, d, order, emb_dim) + tuple(v for r in rows for v in r) + tuple(skip_row)
+        dev = keep[0].device
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("a filter pointer table cannot be built during a stream capture: run one forward "
+                               "with these parameter tensors before capturing")
+        self.table = torch.tensor(rows, dtype=torch.int64).to(dev)
+        self.skip = torch.tensor(skip_row, dtype=torch.int64).to(dev)
+
+    def spectrum_floats(self) -> int:
+        return lib.m2_filter_spectrum_bytes(self.d, self.L) // 4
+
+
+def mixer_filter_spectra(table: FilterTable, w_mod: float = 1.0, shift: float = 0.0, first: int = 0,
+                         count: Optional[int] = None, out: Optional[Tensor] = None) -> Tensor:
+    """Spectra (count, m2_filter_spectrum_bytes / 4) fp32 of the mixers [first, first + count) of `table`, generated
+    from the filter parameters in a few launches for all of them (m2_mixer_filters_fwd)."""
+    count = table.nmixers - first if count is None else count
+    if first < 0 or count < 1 or first + count > table.nmixers:
+        raise ValueError(f"mixers [{first}, {first + count}) outside the table of {table.nmixers}")
+    dev = table.table.device
+    n = table.spectrum_floats()
+    if out is None:
+        out = torch.empty(count, n, dtype=torch.float32, device=dev)
+    else:
+        _require(out, "out", torch.float32, (count, n))
+    ws_bytes = lib.m2_mixer_filters_workspace_bytes(count, table.fpm, table.L, table.d, table.order)
+    workspace = torch.empty((ws_bytes + 3) // 4, dtype=torch.float32, device=dev)
+    check(lib.m2_mixer_filters_fwd(ctypes.c_void_p(table.table.data_ptr() + first * table.fpm * 18 * 8),
+                                   ctypes.c_void_p(table.skip.data_ptr() + first * table.fpm * 8), count, table.fpm,
+                                   table.L, table.d, table.order, table.emb_dim, float(w_mod), float(shift),
+                                   _ptr(workspace), _ptr(out), _stream()))
+    return out
+
+
 def filter_spectrum(taps1: Tensor, taps2: Optional[Tensor], D1: Optional[Tensor], D2: Optional[Tensor]) -> Tensor:
     """Opaque spectrum buffer for `mixer_core` from (d, 2L) taps of one or two filters."""
     d, n = taps1.shape

@@ -54,6 +54,53 @@ def test_hyena_filter_taps(gpu, L, std):
         assert rel_err(hr.cpu(), kr.T[None])[0] < max(2e-5, 4 * e32)
 
 
+@pytest.mark.parametrize("L", [128, 256, 512, 1024, 2048])
+@pytest.mark.parametrize("bidirectional,residual", [(True, True), (False, True), (True, False)])
+def test_mixer_filter_spectra_batched(gpu, L, bidirectional, residual):
+    """m2_mixer_filters_fwd (all filters of three mixers -> spectra in one call; for L <= 512 projection, decay and
+    transform are one kernel and the taps never exist) against the fp64 oracle's taps pushed through the stand-alone
+    spectrum kernel, with the two-step path (m2_hyena_filter_fwd + m2_filter_spectrum_fwd, itself pinned against the
+    oracle above) as the yardstick; also sub-ranges of the table."""
+    import m2_amd
+    from m2_amd import ops
+    from oracle import m2_oracle as O
+    d, nm = 192, 3
+    mixers, sds = [], []
+    for i in range(nm):
+        cfg = _cfg(L, d=d)
+        cfg.bidirectional, cfg.residual_long_conv = bidirectional, residual
+        sd = m2_amd.seeded_state_dict(cfg, 70 + i, std=0.1, what="mixer")
+        mix = m2_amd.MonarchMixerSequenceMixing(d, l_max=L, bidirectional=bidirectional, hyena_emb_dim=5,
+                                                hyena_filter_order=128, residual_long_conv=residual, hyena_w=10)
+        mix.load_state_dict(sd)
+        mixers.append(mix.to(gpu))
+        sds.append(sd)
+    entries = [m.filter_table_entry() for m in mixers]
+    table = ops.FilterTable([e[0] for e in entries], [e[1] for e in entries], L, d, 128, 5)
+    got = ops.mixer_filter_spectra(table)
+    assert got.shape == (nm, ops.lib.m2_filter_spectrum_bytes(d, L) // 4)
+    names = ["filter_fn."] + (["filter_fn2."] if residual else [])
+    for i, (mix, sd) in enumerate(zip(mixers, sds)):
+        sd64 = O.cast_state_dict(sd, torch.float64)
+        taps64, taps_gpu = [], []
+        for name in names:
+            kf = O.hyena_filter_taps(sd64, name, L, rev=False)[0].T
+            kr = O.hyena_filter_taps(sd64, name, L, rev=True)[0].T if bidirectional else torch.zeros_like(kf)
+            taps64.append(O.bidirectional_kernel(kf, kr, L).float().to(gpu).contiguous())
+        fns = [mix.filter_fn] + ([mix.filter_fn2] if residual else [])
+        taps_gpu = [f.bidirectional_taps(L) for f in fns]
+        D = [f.bias.detach().float() for f in fns]
+        want = ops.filter_spectrum(taps64[0], taps64[1] if residual else None, D[0], D[1] if residual else None)
+        two_step = ops.filter_spectrum(taps_gpu[0], taps_gpu[1] if residual else None, D[0], D[1] if residual else None)
+        e, e2 = rel_err(got[i], want)
+        y, _ = rel_err(two_step, want)
+        assert e < max(2e-5, 3 * y), (i, e, e2, y)
+    # a sub-range of the table, into a caller's buffer
+    part = torch.full((2, got.shape[1]), float("nan"), device=gpu)
+    assert ops.mixer_filter_spectra(table, first=1, count=2, out=part) is part
+    assert torch.equal(part, got[1:])
+
+
 @pytest.mark.parametrize("L", [8192, 32768])
 def test_hyena_filter_taps_at_benchmark_lengths(gpu, L):
     """Filter taps at the benchmark's own sizes (d = 768, L = 8192 and 32768: the 64-position hidden tiles and the
@@ -326,14 +373,21 @@ def test_encoder_overlapped_filter_generation_matches_sequential(gpu):
     model.load_state_dict(m2_amd.seeded_state_dict(cfg, 43))
     model = model.to(gpu).eval()
     ids = torch.randint(0, cfg.vocab_size, (2, 256), generator=torch.Generator().manual_seed(10)).to(gpu)
-    model.encoder.overlap_filters = False          # in line on the main stream
-    want, _ = model(ids)
-    for mode in (True, "upfront", None):            # None picks "upfront" at this length
-        model.encoder.overlap_filters = mode
-        for _ in range(3):
-            got, _ = model(ids)
-            torch.cuda.synchronize()
-            assert torch.equal(got, want), mode
+    for batch in (True, False):                     # all layers' filters by batched calls / layer by layer
+        model.encoder.batch_filters = batch
+        model.encoder.overlap_filters = False          # on the main stream
+        want, _ = model(ids)
+        for mode in (True, "upfront", None):            # None picks "upfront" at this length
+            model.encoder.overlap_filters = mode
+            for _ in range(3):
+                got, _ = model(ids)
+                torch.cuda.synchronize()
+                assert torch.equal(got, want), (batch, mode)
+        if batch:
+            batched = want
+    # at this length the batched path runs projection + transform as one kernel: same numbers to fp32 rounding
+    assert rel_err(batched, want)[0] < 1e-4
+    model.encoder.batch_filters = True
     # and inside a captured graph (the side stream becomes a parallel branch), replayed with eager work between
     graphed = m2_amd.BertModel(cfg, use_hip_graph=True)
     graphed.load_state_dict(m2_amd.seeded_state_dict(cfg, 43))
