@@ -36,6 +36,7 @@
 #include <stdint.h>
 
 #include "fft_engine.h"
+#include "hyena_filter.h"
 #include "row_io.h"
 
 namespace m2 {
@@ -226,18 +227,23 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
 // ------------------------------------------------------------------------------------------
 template <class P>
 __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
-    const float* __restrict__ taps1,    // (d, N) bidirectional taps of filter_fn
-    const float* __restrict__ taps2,    // (d, N) bidirectional taps of filter_fn2 (may be null)
-    const float* __restrict__ D1,       // (d) skip weight of filter_fn, added to tap 0 (may be null)
-    const float* __restrict__ D2,       // (d) skip weight of filter_fn2 (may be null)
+    const float* taps1,    // (d, N) bidirectional taps of filter_fn
+    const float* taps2,    // (d, N) bidirectional taps of filter_fn2 (may be null)
+    const float* D1,       // (d) skip weight of filter_fn, added to tap 0 (may be null)
+    const float* D2,       // (d) skip weight of filter_fn2 (may be null)
     float4* __restrict__ spec,          // (d, 8, T)
-    int d) {
+    int d, SpectrumBatch sb) {
   constexpr int N = P::N, T = P::T;
   extern __shared__ float2 lds[];
   const int tid = threadIdx.x;
   const int rloc = tid / T, t = tid % T;
   float2* row = lds + rloc * P::ROW_LDS;
   const int n0 = 16 * t;
+  {
+    float* sp = reinterpret_cast<float*>(spec);
+    select_mixer(sb, d, N, taps1, taps2, D1, D2, sp);
+    spec = reinterpret_cast<float4*>(sp);
+  }
 
   Twiddles<P> tw;
   twiddles_init<P>(tw, t, lds + P::RPW * P::ROW_LDS);
@@ -271,33 +277,7 @@ __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
     forward_to_pairs<P, false>(x, t, row, tw, g, g2);
     row_sync<P>();      // LDS is reused by the next row
 
-    float4 K[8];
-    auto split = [&](cf za, cf zb) -> float4 {
-      // K1 = (za + conj zb) * scale ; K2 = (za - conj zb) / i * scale
-      return make_float4(scale * (za.re + zb.re), scale * (za.im - zb.im), scale * (za.im + zb.im),
-                         scale * (zb.re - za.re));
-    };
-    if (t != 0) {
-      static_for<0, 8>([&](auto jj) {
-        constexpr int j = decltype(jj)::value;
-        K[j] = split(x[bitrev(j, 3)], x[8 + bitrev(7 - j, 3)]);
-      });
-    } else {
-      const cf z0 = x[bitrev(0, 3)], z4 = x[bitrev(4, 3)];
-      K[0] = make_float4(2.f * scale * z0.re, 2.f * scale * z4.re, 2.f * scale * z0.im, 2.f * scale * z4.im);
-      static_for<1, 4>([&](auto jj) {
-        constexpr int j = decltype(jj)::value;
-        K[j] = split(x[bitrev(j, 3)], x[bitrev(8 - j, 3)]);
-      });
-      static_for<0, 4>([&](auto jj) {
-        constexpr int j = decltype(jj)::value;
-        K[4 + j] = split(x[8 + bitrev(j, 3)], x[8 + bitrev(7 - j, 3)]);
-      });
-    }
-    if (valid) {
-      float4* sp = spec + (long)c * 8 * T + t;
-      static_for<0, 8>([&](auto s) { sp[decltype(s)::value * T] = K[decltype(s)::value]; });
-    }
+    if (valid) store_filter_spectrum<P>(x, t, scale, spec + (long)c * 8 * T + t);
   }
 }
 
@@ -338,7 +318,7 @@ static int launch_mixer_core(const void* xproj, const float* u, const float* sw,
 
 template <class P>
 static int launch_filter_spectrum(const float* taps1, const float* taps2, const float* D1, const float* D2,
-                                  float* spec, int d, hipStream_t stream) {
+                                  float* spec, int d, const SpectrumBatch& sb, int nmixers, hipStream_t stream) {
   const size_t lds_bytes = (size_t)P::WG_LDS * sizeof(float2);
   auto kern = filter_spectrum_kernel<P>;
   if (lds_bytes > 64 * 1024) {
@@ -348,7 +328,7 @@ static int launch_filter_spectrum(const float* taps1, const float* taps2, const 
   const int wgs_needed = (d + P::RPW - 1) / P::RPW;
   int grid = num_cus() * 2;
   if (grid > wgs_needed) grid = wgs_needed;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(P::WG), lds_bytes, stream, taps1, taps2, D1, D2, (float4*)spec, d);
+  hipLaunchKernelGGL(kern, dim3(grid, nmixers), dim3(P::WG), lds_bytes, stream, taps1, taps2, D1, D2, (float4*)spec, d, sb);
   return check_launch("filter_spectrum");
 }
 
@@ -364,14 +344,30 @@ size_t real_spectrum_bytes(int d);
 int launch_mixer_real_dispatch(const void* xproj, const float* u, const float* sw, const float* sb, const float* pbias,
                                const float* spec, void* y, int B, int d, int act_dtype, hipStream_t stream);
 int launch_filter_spectrum_real(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
-                                int d, hipStream_t stream);
+                                int d, const SpectrumBatch& sb, int nmixers, hipStream_t stream);
 
 // L = 2048 .. 16384: even/odd split half transforms, defined in fftconv_split_kernels.hip
 bool split_plan_exists(int L);
 int launch_mixer_split_dispatch(const void* xproj, const float* u, const float* sw, const float* sb, const float* pbias,
                                 const float* spec, void* y, int B, int L, int d, int act_dtype, hipStream_t stream);
 int launch_filter_spectrum_split(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
-                                 int d, int L, hipStream_t stream);
+                                 int d, int L, const SpectrumBatch& sb, int nmixers, hipStream_t stream);
+
+// One mixer given by pointers (sb.taps null, nmixers 1) or a batch of mixers described by `sb`.
+int launch_filter_spectrum_any(const float* taps1, const float* taps2, const float* D1, const float* D2, float* spec,
+                               int d, int L, const SpectrumBatch& sb, int nmixers, hipStream_t stream) {
+  const int logn = ilog2(2 * L);
+  if (logn == 16) return launch_filter_spectrum_real(taps1, taps2, D1, D2, spec, d, sb, nmixers, stream);
+  if (split_plan_exists(L)) return launch_filter_spectrum_split(taps1, taps2, D1, D2, spec, d, L, sb, nmixers, stream);
+  switch (logn) {
+#define X(LOGN, R1, R2, R3) \
+  case LOGN:                \
+    return launch_filter_spectrum<Plan<LOGN, R1, R2, R3>>(taps1, taps2, D1, D2, spec, d, sb, nmixers, stream);
+    M2_FOR_EACH_PLAN(X)
+#undef X
+  }
+  return set_error(M2_ERR_UNSUPPORTED, "filter spectrum: no plan for L=%d", L);
+}
 
 }  // namespace m2
 
@@ -393,17 +389,8 @@ extern "C" int m2_filter_spectrum_fwd(const float* taps1, const float* taps2, co
   if (d <= 0) return set_error(M2_ERR_ARG, "m2_filter_spectrum_fwd: d must be positive, got %d", d);
   if (!m2_fftconv_supported_seqlen(L))
     return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: L=%d unsupported (need L a power of two in [128, 32768])", L);
-  const int logn = ilog2(2 * L);
-  if (logn == 16) return launch_filter_spectrum_real(taps1, taps2, D1, D2, spec, d, (hipStream_t)stream);
-  if (split_plan_exists(L)) return launch_filter_spectrum_split(taps1, taps2, D1, D2, spec, d, L, (hipStream_t)stream);
-  switch (logn) {
-#define X(LOGN, R1, R2, R3) \
-  case LOGN:                \
-    return launch_filter_spectrum<Plan<LOGN, R1, R2, R3>>(taps1, taps2, D1, D2, spec, d, (hipStream_t)stream);
-    M2_FOR_EACH_PLAN(X)
-#undef X
-  }
-  return set_error(M2_ERR_UNSUPPORTED, "m2_filter_spectrum_fwd: no plan for L=%d", L);
+  const SpectrumBatch none{nullptr, nullptr, 0, 0};
+  return launch_filter_spectrum_any(taps1, taps2, D1, D2, spec, d, L, none, 1, (hipStream_t)stream);
 }
 
 extern "C" int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, const float* u, const float* short_w,
