@@ -29,7 +29,19 @@ struct Plan {
   static constexpr int RL = (R3 > 1) ? R3 : R2;   // radix of the least significant digit of a group index
   static constexpr int WG = T < 256 ? 256 : T;    // threads per workgroup
   static constexpr int RPW = WG / T;              // rows per workgroup
-  static constexpr int ROW_LDS = N + (N >> 4);    // padded complex slots per row
+  // LDS layout of a row: slot of position p is p + PA (p >> SA) + PB (p >> SB); PX more slots end the row.  All pads
+  // are even numbers of 8-byte slots, so 16-byte accesses stay aligned; the values per length come from enumerating
+  // the 64 banks for every access pattern of the plan (staging, the strided passes, the contiguous groups) with the
+  // rows a wavefront holds side by side.
+  static constexpr int SA = LOGN_ == 8 ? 4 : 5, PA = 2;
+  static constexpr int SB = LOGN_ == 8 ? 7 : LOGN_ == 9 ? 8 : LOGN_ == 10 ? 7 : 9;
+  static constexpr int PB = LOGN_ == 8 ? 4 : LOGN_ == 11 ? 4 : 2;
+  static constexpr int PX = LOGN_ == 8 ? 8 : 0;
+  __host__ __device__ static constexpr int phys(int pos) { return pos + PA * (pos >> SA) + PB * (pos >> SB); }
+  // Padded offset of logical offset `o` relative to a base position, valid where adding `o` to the base carries into
+  // neither bit SA nor bit SB from below (checked for every access of the plan by plan_offsets_ok).
+  __host__ __device__ static constexpr int poff(int o) { return o + PA * (o >> SA) + PB * (o >> SB); }
+  static constexpr int ROW_LDS = N + PA * (N >> SA) + PB * (N >> SB) + PX;    // padded complex slots per row
   static constexpr int TW_LDS = R2 * (N / R1 / R2) + (R3_ > 1 ? R3_ * (N / R1 / R2 / R3_) : 0);   // twiddle tables
   static constexpr int WG_LDS = (T < 256 ? 256 / T : 1) * ROW_LDS + TW_LDS;                         // float2 slots per workgroup
   static_assert(R1 * R2 * R3 * RP == N, "radices must multiply to N");
@@ -37,12 +49,30 @@ struct Plan {
   static_assert(R1 * R2 >= E, "passes after the first must share twiddles inside a thread");
 };
 
-__device__ __forceinline__ int phys(int pos) { return pos + (pos >> 4); }
-
-// Padded offset of logical offset `o` relative to a base position whose low four bits, added to
-// (o mod 16), stay below 16.  True for every access below: strides are multiples of 16, or 8 with a
-// base offset below 8, or consecutive runs of 8 that start at a multiple of 8.
-constexpr int poff(int o) { return o + (o >> 4); }
+// phys(base + o) == phys(base) + poff(o) for every (base, offset) pair the passes of plan P use: the strided passes
+// (base = the thread's butterfly position, o = j S) and the runs of 8 / 16 consecutive slots of staging and of the
+// last pass.
+template <class P>
+constexpr bool plan_offsets_ok() {
+  for (int q = 0; q < P::N / P::R1; ++q)
+    for (int j = 0; j < P::R1; ++j)
+      if (P::phys(q + j * P::S1) != P::phys(q) + P::poff(j * P::S1)) return false;
+  for (int q = 0; q < P::N / P::R2; ++q) {
+    const int base = (q / P::S2) * (P::S2 * P::R2) + q % P::S2;
+    for (int j = 0; j < P::R2; ++j)
+      if (P::phys(base + j * P::S2) != P::phys(base) + P::poff(j * P::S2)) return false;
+  }
+  if (P::R3 > 1)
+    for (int q = 0; q < P::N / P::R3; ++q) {
+      const int base = (q / P::S3) * (P::S3 * P::R3) + q % P::S3;
+      for (int j = 0; j < P::R3; ++j)
+        if (P::phys(base + j * P::S3) != P::phys(base) + P::poff(j * P::S3)) return false;
+    }
+  for (int g = 0; g < P::N / 16; ++g)
+    for (int j = 0; j < 16; ++j)
+      if (P::phys(16 * g + j) != P::phys(16 * g) + j) return false;
+  return P::ROW_LDS % 2 == 0 && P::phys(P::N - 1) < P::ROW_LDS;
+}
 
 __device__ __forceinline__ cf lds_get(const float2* p, int off) {
   float2 v = p[off];
@@ -138,7 +168,7 @@ __device__ __forceinline__ void fwd_compute_store(cf (&x)[16], int t, float2* ro
     const int b = q / S, m = q % S;
     if constexpr (ZERO_UPPER) dif_zero_upper<R, i * R, 16>(x);
     else dif<R, i * R, 16>(x);
-    float2* pb = row + phys(b * (S * R) + m);
+    float2* pb = row + P::phys(b * (S * R) + m);
     constexpr int bits = ilog2(R);
     cf pw[PASS == 1 ? P::R1 : 1];
     if constexpr (PASS == 1) pass1_twiddles<P, i>(tw, pw);
@@ -149,7 +179,7 @@ __device__ __forceinline__ void fwd_compute_store(cf (&x)[16], int t, float2* ro
         if constexpr (PASS == 1) v = cmul(v, pw[k]);
         else v = cmul(v, table_twiddle<P, PASS, S, k>(tw, m));
       }
-      lds_put(pb, poff(k * S), v);
+      lds_put(pb, P::poff(k * S), v);
     });
   });
 }
@@ -161,10 +191,10 @@ __device__ __forceinline__ void fwd_load(cf (&x)[16], int t, const float2* row) 
     constexpr int i = decltype(ii)::value;
     const int q = t + P::T * i;
     const int b = q / S, m = q % S;
-    const float2* pb = row + phys(b * (S * R) + m);
+    const float2* pb = row + P::phys(b * (S * R) + m);
     static_for<0, R>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
-      x[i * R + j] = lds_get(pb, poff(j * S));
+      x[i * R + j] = lds_get(pb, P::poff(j * S));
     });
   });
 }
@@ -177,13 +207,13 @@ __device__ __forceinline__ void inv_load_compute(cf (&x)[16], int t, const float
     constexpr int i = decltype(ii)::value;
     const int q = t + P::T * i;
     const int b = q / S, m = q % S;
-    const float2* pb = row + phys(b * (S * R) + m);
+    const float2* pb = row + P::phys(b * (S * R) + m);
     constexpr int bits = ilog2(R);
     cf pw[PASS == 1 ? P::R1 : 1];
     if constexpr (PASS == 1) pass1_twiddles<P, i>(tw, pw);
     static_for<0, R>([&](auto kk) {
       constexpr int k = decltype(kk)::value;
-      cf v = lds_get(pb, poff(k * S));
+      cf v = lds_get(pb, P::poff(k * S));
       if constexpr (k > 0) {
         if constexpr (PASS == 1) v = cmulc(v, pw[k]);
         else v = cmulc(v, table_twiddle<P, PASS, S, k>(tw, m));
@@ -202,10 +232,10 @@ __device__ __forceinline__ void inv_store(const cf (&x)[16], int t, float2* row)
     constexpr int i = decltype(ii)::value;
     const int q = t + P::T * i;
     const int b = q / S, m = q % S;
-    float2* pb = row + phys(b * (S * R) + m);
+    float2* pb = row + P::phys(b * (S * R) + m);
     static_for<0, R>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
-      lds_put(pb, poff(j * S), x[i * R + j]);
+      lds_put(pb, P::poff(j * S), x[i * R + j]);
     });
   });
 }
@@ -247,8 +277,8 @@ __device__ __forceinline__ void forward_to_pairs(cf (&x)[16], int t, float2* row
     row_sync<P>();
   }
   {
-    const float2* pa = row + phys(g * 8);
-    const float2* pb = row + phys(g2 * 8);
+    const float2* pa = row + P::phys(g * 8);
+    const float2* pb = row + P::phys(g2 * 8);
     static_for<0, 8>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
       x[j] = lds_get(pa, j);
@@ -278,8 +308,8 @@ __device__ __forceinline__ void inverse_from_pairs(cf (&x)[16], int t, float2* r
   dit<8, 0, 16>(x);
   dit<8, 8, 16>(x);
   {
-    float2* pa = row + phys(g * 8);
-    float2* pb = row + phys(g2 * 8);
+    float2* pa = row + P::phys(g * 8);
+    float2* pb = row + P::phys(g2 * 8);
     static_for<0, 8>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
       lds_put(pa, j, x[j]);

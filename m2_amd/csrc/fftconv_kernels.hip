@@ -50,10 +50,10 @@ __device__ __forceinline__ void fwd_load_lower(cf (&x)[16], int t, const float2*
   constexpr int R = P::R1, S = P::S1, NB = 16 / R;
   static_for<0, NB>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
-    const float2* pb = row + phys(t + P::T * i);
+    const float2* pb = row + P::phys(t + P::T * i);
     static_for<0, R / 2>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
-      x[i * R + j] = lds_get(pb, poff(j * S));
+      x[i * R + j] = lds_get(pb, P::poff(j * S));
     });
   });
 }
@@ -62,13 +62,18 @@ __device__ __forceinline__ void inv_store_lower(const cf (&x)[16], int t, float2
   constexpr int R = P::R1, S = P::S1, NB = 16 / R;
   static_for<0, NB>([&](auto ii) {
     constexpr int i = decltype(ii)::value;
-    float2* pb = row + phys(t + P::T * i);
+    float2* pb = row + P::phys(t + P::T * i);
     static_for<0, R / 2>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
-      lds_put(pb, poff(j * S), x[i * R + j]);
+      lds_put(pb, P::poff(j * S), x[i * R + j]);
     });
   });
 }
+
+// Per-row constants of the short convolutions, staged through LDS: the T threads of a row share one channel, so
+// thread k < 15 of the row fetches constant k and all of them read the set back (one register per thread in
+// flight instead of fifteen).  Order: (w0, w1, w2, conv bias, projection bias) of x1, then of v, then of x2.
+constexpr int kRowConsts = 16;
 
 template <class P, typename ACT>
 __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
@@ -85,6 +90,7 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
   const int tid = threadIdx.x;
   const int rloc = tid / T, t = tid % T;
   float2* row = lds + rloc * P::ROW_LDS;
+  float* crow = reinterpret_cast<float*>(lds + P::RPW * P::ROW_LDS + P::TW_LDS) + rloc * kRowConsts;
   const int n0 = 8 * t;
 
   Twiddles<P> tw;
@@ -97,42 +103,60 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
   // channel's spectrum is fetched into that L2 once and shared.  (d % 8 == 0 is checked by the host.)
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
   const int rows_per_xcd = (d >> 3) * B;
+
+  // The inputs of a row batch are requested one batch ahead: the loads of batch i + 1 are issued as soon as the
+  // registers of batch i have been consumed by its prologue, and travel while batch i is transformed.  Without
+  // this the workgroups of a compute unit, which start together, stay in step: all load, then all compute, and
+  // memory time adds to arithmetic time instead of hiding behind it.
+  RawRow<ACT, 1> r1, r2, rv;
+  f32x4_t u0 = {0.f, 0.f, 0.f, 0.f}, u1 = u0;
+  float cst = 0.f;
+  auto fetch_batch = [&](int j0) __attribute__((always_inline)) {
+    const int j = j0 + rloc;
+    const int jj = j < rows_per_xcd ? j : rows_per_xcd - 1;
+    const int c = (jj / B) * 8 + xcd, b = jj % B;
+    if (sw) {
+      r1.template fetch<0>(xproj + ((long)(0 * d + c) * B + b) * L, n0);
+      rv.template fetch<0>(xproj + ((long)(2 * d + c) * B + b) * L, n0);
+      r2.template fetch<0>(xproj + ((long)(1 * d + c) * B + b) * L, n0);
+      if (t < 15) {
+        const int grp = t / 5, k = t % 5;
+        const long ch = (long)(grp == 0 ? 0 : grp == 1 ? 2 : 1) * d + c;
+        cst = k < 3 ? sw[ch * 3 + k] : k == 3 ? sb[ch] : (pbias ? pbias[ch] : 0.f);
+      }
+    } else {
+      r1.template fetch<0>(xproj + ((long)c * B + b) * L, n0);
+    }
+    if (uin) {
+      const float* pu = uin + ((long)c * B + b) * L + n0;
+      u0 = *reinterpret_cast<const f32x4_t*>(pu);
+      u1 = *reinterpret_cast<const f32x4_t*>(pu + 4);
+    }
+  };
+  if (slot * P::RPW < rows_per_xcd) fetch_batch(slot * P::RPW);
+
   for (int j0 = slot * P::RPW; j0 < rows_per_xcd; j0 += slots * P::RPW) {
     const int j = j0 + rloc;
     const bool valid = j < rows_per_xcd;
     const int jj = valid ? j : rows_per_xcd - 1;
     const int c = (jj / B) * 8 + xcd, b = jj % B;
 
-    // ---- prologue: 8 consecutive time steps per thread: short conv, gate, stage z = a + i u in LDS.  All loads of
-    // the row are put in flight before the first is converted (one memory latency per row, not one per signal) ----
-    float gate[8];
+    // ---- prologue: 8 consecutive time steps per thread: short conv, gate, stage z = a + i u in LDS ----
+    GateRow<ACT, 1> gate;
     {
-      float in[10], a[8];
-      RawRow<ACT, 1> r1, r2, rv;
-      f32x4_t u0 = {0.f, 0.f, 0.f, 0.f}, u1 = u0;
+      float in[10], a[8], gt[8];
       if (sw) {
-        r1.template fetch<0>(xproj + ((long)(0 * d + c) * B + b) * L, n0);
-        rv.template fetch<0>(xproj + ((long)(2 * d + c) * B + b) * L, n0);
-        r2.template fetch<0>(xproj + ((long)(1 * d + c) * B + b) * L, n0);
-      } else {
-        r1.template fetch<0>(xproj + ((long)c * B + b) * L, n0);
-      }
-      if (uin) {
-        const float* pu = uin + ((long)c * B + b) * L + n0;
-        u0 = *reinterpret_cast<const f32x4_t*>(pu);
-        u1 = *reinterpret_cast<const f32x4_t*>(pu + 4);
-      }
-      if (sw) {
-        const float* w = sw + (long)c * 3;
-        const float w10 = w[0], w11 = w[1], w12 = w[2], bb1 = sb[c];
-        const float wv0 = w[6 * (long)d + 0], wv1 = w[6 * (long)d + 1], wv2 = w[6 * (long)d + 2], bbv = sb[2 * d + c];
-        const float w20 = w[3 * (long)d + 0], w21 = w[3 * (long)d + 1], w22 = w[3 * (long)d + 2], bb2 = sb[d + c];
-        const float p1 = pbias ? pbias[c] : 0.f, pv = pbias ? pbias[2 * d + c] : 0.f, p2 = pbias ? pbias[d + c] : 0.f;
+        if (t < 15) crow[t] = cst;
+        row_sync<P>();
+        const float4 c0 = *reinterpret_cast<const float4*>(crow), c1 = *reinterpret_cast<const float4*>(crow + 4),
+                     c2 = *reinterpret_cast<const float4*>(crow + 8), c3 = *reinterpret_cast<const float4*>(crow + 12);
+        const float w10 = c0.x, w11 = c0.y, w12 = c0.z, bb1 = c0.w, p1 = c1.x;
+        const float wv0 = c1.y, wv1 = c1.z, wv2 = c1.w, bbv = c2.x, pv = c2.y;
+        const float w20 = c2.z, w21 = c2.w, w22 = c3.x, bb2 = c3.y, p2 = c3.z;
         // The bias p of the in-projection is not added to the inputs: a 3-tap convolution of (x + p) is the
         // convolution of x plus p (w0 + w1 + w2), which goes into the convolution's own bias -- except for the first
         // two outputs of a row, where one or two taps fall on the zero padding: those are corrected.
         const float f1 = bb1 + p1 * (w10 + w11 + w12), fv = bbv + pv * (wv0 + wv1 + wv2), f2 = bb2 + p2 * (w20 + w21 + w22);
-        __builtin_amdgcn_sched_barrier(0);
         float cv[8];
         r1.template expand<0>(n0, in);
         static_for<0, 8>([&](auto jj) {
@@ -147,12 +171,12 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
         r2.template expand<0>(n0, in);
         static_for<0, 8>([&](auto jj) {
           constexpr int j = decltype(jj)::value;
-          gate[j] = f2 + w20 * in[j] + w21 * in[j + 1] + w22 * in[j + 2];
+          gt[j] = f2 + w20 * in[j] + w21 * in[j + 1] + w22 * in[j + 2];
         });
         if (n0 == 0) {      // time steps 0 and 1 of the row
           a[0] -= p1 * (w10 + w11); a[1] -= p1 * w10;
           cv[0] -= pv * (wv0 + wv1); cv[1] -= pv * wv0;
-          gate[0] -= p2 * (w20 + w21); gate[1] -= p2 * w20;
+          gt[0] -= p2 * (w20 + w21); gt[1] -= p2 * w20;
         }
         static_for<0, 8>([&](auto jj) { a[decltype(jj)::value] *= cv[decltype(jj)::value]; });
       } else {
@@ -161,15 +185,20 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
         static_for<0, 8>([&](auto jj) {
           constexpr int j = decltype(jj)::value;
           a[j] = in[j + 2];
-          gate[j] = 1.f;
+          gt[j] = 1.f;
         });
       }
-      float4* dst = reinterpret_cast<float4*>(row + phys(n0));     // 8 consecutive slots never straddle a pad
+      gate.template set<0>(gt);
+      float4* dst = reinterpret_cast<float4*>(row + P::phys(n0));     // 8 consecutive slots never straddle a pad
       dst[0] = make_float4(a[0], u0.x, a[1], u0.y);
       dst[1] = make_float4(a[2], u0.z, a[3], u0.w);
       dst[2] = make_float4(a[4], u1.x, a[5], u1.y);
       dst[3] = make_float4(a[6], u1.z, a[7], u1.w);
     }
+    // the next batch's loads, behind everything that read this batch's registers
+    __builtin_amdgcn_sched_barrier(0);
+    if (j0 + slots * P::RPW < rows_per_xcd) fetch_batch(j0 + slots * P::RPW);
+    __builtin_amdgcn_sched_barrier(0);
     row_sync<P>();
 
     cf x[16];
@@ -209,13 +238,13 @@ __global__ __launch_bounds__(P::WG) void mixer_core_kernel(
 
     // ---- epilogue: 8 consecutive outputs per thread ----
     {
-      const float4* src = reinterpret_cast<const float4*>(row + phys(n0));
+      const float4* src = reinterpret_cast<const float4*>(row + P::phys(n0));
       const float4 o0 = src[0], o1 = src[1], o2 = src[2], o3 = src[3];
       float out[8];
-      out[0] = o0.x * gate[0] + o0.y; out[1] = o0.z * gate[1] + o0.w;
-      out[2] = o1.x * gate[2] + o1.y; out[3] = o1.z * gate[3] + o1.w;
-      out[4] = o2.x * gate[4] + o2.y; out[5] = o2.z * gate[5] + o2.w;
-      out[6] = o3.x * gate[6] + o3.y; out[7] = o3.z * gate[7] + o3.w;
+      out[0] = o0.x * gate.template get<0>() + o0.y; out[1] = o0.z * gate.template get<1>() + o0.w;
+      out[2] = o1.x * gate.template get<2>() + o1.y; out[3] = o1.z * gate.template get<3>() + o1.w;
+      out[4] = o2.x * gate.template get<4>() + o2.y; out[5] = o2.z * gate.template get<5>() + o2.w;
+      out[6] = o3.x * gate.template get<6>() + o3.y; out[7] = o3.z * gate.template get<7>() + o3.w;
       if (valid) store8(y + ((long)c * B + b) * L, n0, out);
     }
     row_sync<P>();      // the next row's prologue overwrites what the epilogue has just read
@@ -257,7 +286,7 @@ __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
     const int c = valid ? r : d - 1;
     {   // 16 consecutive taps of each filter per thread -> z = k1 + i k2 staged in LDS
       const float4* p1 = reinterpret_cast<const float4*>(taps1 + (long)c * N + n0);
-      float4* dst = reinterpret_cast<float4*>(row + phys(n0));
+      float4* dst = reinterpret_cast<float4*>(row + P::phys(n0));
       static_for<0, 4>([&](auto qq) {
         constexpr int q = decltype(qq)::value;
         float4 a = p1[q];
@@ -287,7 +316,7 @@ __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
 template <class P, typename ACT>
 static int launch_mixer_core(const void* xproj, const float* u, const float* sw, const float* sb, const float* pbias,
                              const float* spec, void* y, int B, int d, hipStream_t stream) {
-  const size_t lds_bytes = (size_t)P::WG_LDS * sizeof(float2);
+  const size_t lds_bytes = (size_t)P::WG_LDS * sizeof(float2) + (size_t)P::RPW * kRowConsts * sizeof(float);
   auto kern = mixer_core_kernel<P, ACT>;
   if (lds_bytes > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -338,6 +367,10 @@ static int launch_filter_spectrum(const float* taps1, const float* taps2, const 
   X(9, 8, 8, 1)             \
   X(10, 16, 8, 1)           \
   X(11, 16, 16, 1)
+
+#define X(LOGN, R1, R2, R3) static_assert(plan_offsets_ok<Plan<LOGN, R1, R2, R3>>(), "LDS offsets of the plan");
+M2_FOR_EACH_PLAN(X)
+#undef X
 
 // L = 32768 (every real signal on its own, as half transforms of 16384 points), defined in fftconv_real_kernels.hip
 size_t real_spectrum_bytes(int d);

@@ -98,7 +98,7 @@ __global__ __launch_bounds__(kFusedRows* P::T) void project_spectrum_kernel(
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[ks], __builtin_bit_cast(bf16x8, bh[ks]), acc, 0, 0, 0);
         // accumulator element j of lane (i16, q4): channel c0 + 4 q4 + j, position p
         const int idx = dir == 0 ? p : N - 1 - p;
-        float* dst = reinterpret_cast<float*>(lds + (4 * q4) * P::ROW_LDS + phys(idx)) + which;
+        float* dst = reinterpret_cast<float*>(lds + (4 * q4) * P::ROW_LDS + P::phys(idx)) + which;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           // exp(-t |delta|); the bare hardware exp2 flushes results below 2^-126 to zero, which is the value to
