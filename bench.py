@@ -45,10 +45,23 @@ import torch
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# HBM-side bytes per mixer-core launch at the default workload, from the two rocprofv3 --pmc runs
-# (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000 against a plain 256 MiB copy); summary in
-# profiles/encoder_fwd_L8192_B4_hbm_traffic.md.  Only valid for --config c3.
-MIXER_CORE_TRAFFIC_BYTES_C3 = int((190182 * 2.0 + 55629 * 1.0) * 1024)
+# HBM-side bytes per mixer-core launch at the default workload: not measured by the run that prints it (counters need
+# rocprofv3) but by the two --pmc runs summarised in profiles/encoder_fwd_L8192_B4_hbm_traffic.md (FETCH_SIZE scaled
+# by 2.000, WRITE_SIZE by 1.000 against a plain 256 MiB copy).  Stamped with the state of the kernel it was taken
+# from; reported only for --config c3, with the stamp beside it.
+MIXER_CORE_TRAFFIC_C3 = {"bytes": int((190182 * 2.0 + 55629 * 1.0) * 1024), "kernel": "mixer_split_kernel",
+                         "measured": "2026-11-24", "commit": "2847b0b",
+                         "source": "profiles/encoder_fwd_L8192_B4_hbm_traffic.md"}
+
+
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 REFERENCE_GRID = {"l512": (512, 32), "l1024": (1024, 32), "l2048": (2048, 16), "l4096": (4096, 8)}
@@ -146,7 +159,7 @@ def cpu_baseline(sd, cfg, ids, mask, B):
     times.sort()
     dt = times[1]
     return ref, {"value": B / dt, "unit": "seq/s", "cores": torch.get_num_threads(), "kind": "port",
-                 "host_cpu_count": os.cpu_count(),
+                 "host_cpu_count": os.cpu_count(), "cpu_model": cpu_model(),
                  "sample": f"full forward (embeddings + {cfg.num_hidden_layers} layers) of the same batch, fp32 "
                            f"torch.fft/einsum oracle: 1 warm-up + 3 timed, median {dt:.2f} s "
                            f"(min {times[0]:.2f}, max {times[2]:.2f})"}
@@ -326,7 +339,8 @@ def main():
                                " with the filter-generation kernels of the layer",
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": MIXER_CORE_TRAFFIC_BYTES_C3 if args.config == "c3" else None,
+                     "traffic": MIXER_CORE_TRAFFIC_C3["bytes"] if args.config == "c3" else None,
+                     "traffic_measured": MIXER_CORE_TRAFFIC_C3 if args.config == "c3" else None,
                      "bytes_per_launch": nbytes, "ms_per_launch": t_core + t_filt, "launches_timed": n_core,
                      "core_only_ms_per_launch": t_core, "core_only_achieved": core_only,
                      "core_only_frac": core_only / HBM_PEAK_GBPS,

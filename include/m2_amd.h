@@ -79,12 +79,13 @@ int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int 
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The intermediate activations
  * go through a device array of M2_HYENA_FILTER_STATIC_SCRATCH_BYTES that is part of the library itself (every GPU
  * the library runs on holds one copy until the process ends); the call allocates and frees nothing.  Limit:
- * m2_hyena_filter_workspace_bytes(nfilters, L, d, order) must not exceed that size, which at d = 768 means
- * nfilters * L <= 16384 (both filters of a mixer up to L = 8192); beyond it the call fails with M2_ERR_UNSUPPORTED.  All calls on one GPU share
+ * m2_hyena_filter_workspace_bytes(nfilters, L, d, order) must not exceed that size: 20 MiB holds nfilters * L <= 16384
+ * for every d <= 1536 (both filters of a mixer up to L = 8192 at d = 768 need 19,136,512 bytes, at d = 1536
+ * 20,709,376); beyond it the call fails with M2_ERR_UNSUPPORTED.  All calls on one GPU share
  * the array: two such calls whose kernels may overlap on the same GPU (different streams, or different host threads
  * on different streams) race; calls on one stream are ordered and safe.  The first call on a device looks up the
  * array's device address (hipGetSymbolAddress): make that call outside a stream capture. */
-#define M2_HYENA_FILTER_STATIC_SCRATCH_BYTES (18u << 20)
+#define M2_HYENA_FILTER_STATIC_SCRATCH_BYTES (20u << 20)
 int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, int nfilters, int L, int d, int order,
                                int emb_dim, float w_mod, float shift, float* taps, void* stream);
 

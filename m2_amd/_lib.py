@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libm2_amd.so")
 
 M2_DTYPE_F32 = 0
 M2_DTYPE_BF16 = 1
-M2_HYENA_FILTER_STATIC_SCRATCH_BYTES = 18 << 20
+M2_HYENA_FILTER_STATIC_SCRATCH_BYTES = 20 << 20
 
 
 class HyenaFilterParams(ctypes.Structure):

@@ -59,7 +59,8 @@ def hyena_filter_taps(filters: Sequence[dict], L: int, d: int, order: int, emb_d
     Each entry is a dict with fp32 GPU tensors: z (>=L, emb), t (>=L), freq (order), deltas (d),
     `fwd` = [w0, b0, w1, b1, w2, b2, w3] and optionally `rev` = the same seven of the reverse MLP.
     `static_scratch=True` takes the library's allocation-free entry point (m2_hyena_filter_fwd_static: no
-    workspace tensor, nfilters * L <= 16384); with `out` given as well nothing is allocated at all.
+    workspace tensor; the 20 MiB static array holds nfilters * L <= 16384 for d <= 1536); with `out` given as well
+    nothing is allocated at all.
     """
     nf = len(filters)
     arr = (HyenaFilterParams * nf)()

@@ -21,18 +21,22 @@ def test_static_scratch_entry_point_matches_workspace_entry_point(gpu):
     import m2_amd
     from m2_amd import ops
     from m2_amd._lib import M2_HYENA_FILTER_STATIC_SCRATCH_BYTES, lib
-    d = 192
+    d = 768                                       # the benchmark's own width: both filters of a mixer at L = 8192
     cfg = m2_amd.m2_bert_80m(8192)
-    cfg.hidden_size = d
     filters, _ = _filters(cfg, 3, gpu)
     for L in (8192, 1024):                       # the second call is shorter: stale scratch beyond it must not matter
         assert lib.m2_hyena_filter_workspace_bytes(2, L, d, 128) <= M2_HYENA_FILTER_STATIC_SCRATCH_BYTES
         want = ops.hyena_filter_taps(filters, L, d, 128, 5)
         out = torch.full((2, d, 2 * L), float("nan"), device=gpu)
+        torch.cuda.synchronize()
         free_before = torch.cuda.mem_get_info()[0]
+        stats_before = torch.cuda.memory_stats()
         got = ops.hyena_filter_taps(filters, L, d, 128, 5, static_scratch=True, out=out)
         torch.cuda.synchronize()
-        assert torch.cuda.mem_get_info()[0] == free_before           # no device allocation behind the call
+        stats_after = torch.cuda.memory_stats()
+        assert torch.cuda.mem_get_info()[0] == free_before           # no device allocation behind the call ...
+        for key in ("allocation.all.allocated", "allocated_bytes.all.allocated", "segment.all.allocated"):
+            assert stats_after[key] == stats_before[key], key         # ... and none served from torch's cache either
         assert got is out and torch.equal(got, want), L
     # against the oracle as well (fp64), the shorter length
     from conftest import rel_err
@@ -44,7 +48,6 @@ def test_static_scratch_entry_point_matches_workspace_entry_point(gpu):
     assert rel_err(got[0], O.bidirectional_kernel(kf, kr, 1024))[0] < 2e-5
     # two filters of 16384 positions do not fit the static array: refused, nothing launched
     cfg_long = m2_amd.m2_bert_80m(16384)
-    cfg_long.hidden_size = d
     long_filters, _ = _filters(cfg_long, 3, gpu)
     with pytest.raises(RuntimeError, match="static array"):
         ops.hyena_filter_taps(long_filters, 16384, d, 128, 5, static_scratch=True)
