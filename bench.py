@@ -172,6 +172,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--reps", type=int, default=5, help="how many times the K timed steps are repeated (median reported)")
     ap.add_argument("--config", default="c3")
+    ap.add_argument("--filters", default="default", choices=["default", "inline", "overlap"],
+                    help="where the timed forward generates its filters: ahead of the layers on the main stream "
+                         "(inline), beside them on a second stream (overlap), or the encoder's own default")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", dest="hip_graph", action="store_false",
                     help="time the eager launches (with the per-launch HIP events in between) instead of the "
@@ -229,10 +232,32 @@ def main():
                                                   "embed_layernorm")
              if timer.count(tag)}
     n_core = timer.count("mixer_core")
-    # filter generation runs as a few launches for ALL layers (one library call per group of layers): per layer
-    # = everything those calls took, divided by the layers they served
-    filt_calls = timer.count("filter_generation")
-    means["filter_generation"] = timer.mean_ms("filter_generation") * filt_calls / max(1, n_core)
+    # Filter generation runs as a few launches for ALL layers (one library call per group of layers).  Inside a
+    # forward those launches sit at the head of an almost empty queue, so an event pair around them also times the
+    # host's launch latency; the kernels' own time is taken from the same calls issued back to back (events around
+    # K repetitions of the whole generation, nothing else on the chip), divided by the layers they serve.
+    plan = model.encoder._batched_filter_plan(L)
+    if plan is not None:
+        table, groups = plan
+        f0 = model.encoder.layer[0].attention.filter_fn
+
+        def generate_all():
+            for first, count in groups:
+                ops.mixer_filter_spectra(table, w_mod=float(f0.w_mod), shift=float(f0.modulation.shift), first=first,
+                                         count=count)
+        with torch.no_grad():
+            generate_all()
+            torch.cuda.synchronize()
+            s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s_ev.record()
+            for _ in range(args.steps):
+                generate_all()
+            e_ev.record()
+            torch.cuda.synchronize()
+        means["filter_generation"] = s_ev.elapsed_time(e_ev) / args.steps / cfg.num_hidden_layers
+        means["filter_generation_in_forward"] = timer.mean_ms("filter_generation") * timer.count("filter_generation") / max(1, n_core)
+    else:
+        means["filter_generation"] = timer.mean_ms("filter_generation") * timer.count("filter_generation") / max(1, n_core)
     for fn, orig in wrapped.items():            # per-launch events are only wanted for the eager timed steps
         setattr(ops, fn, orig)
 
@@ -243,7 +268,7 @@ def main():
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 
-    model.encoder.overlap_filters = None       # the default: filter generation of all layers on a second stream
+    model.encoder.overlap_filters = {"default": None, "inline": False, "overlap": "upfront"}[args.filters]
     if args.hip_graph:
         model.encoder.use_hip_graph = True
     with torch.no_grad():

@@ -107,11 +107,20 @@ constexpr int kActRowB = 2 * kOrder + 16;     // bytes per padded bf16 row of an
 // weights pre-split by split_weights_kernel and held in registers for all tiles (fetching them is what a short run
 // of positions per workgroup pays most for: 96 KB per workgroup and layer from L2).  Within a layer the products of
 // tile i + 1 are issued together with the sin epilogue of tile i, so that matrix pipe and vector ALU overlap.
-template <int TILES, class TAB>
-__global__ __launch_bounds__(256) void hidden_kernel(TAB tab, int L, int emb, float w_mod,
+//
+// PROJECT = true: the same workgroup goes on to the 128 -> d output projection of its positions (the last hidden
+// layer's activations stay in LDS as bf16 hi / lo parts instead of travelling through memory): wave w takes the
+// 32-channel tiles w, w + 4, ..., fetches the tile's pre-split weight rows (hi / lo parts in operand layout, from L2:
+// every workgroup reads all of them once), multiplies (three products: W_hi h_hi + W_hi h_lo + W_lo h_hi), applies
+// exp(-t |delta|) + shift and stores the taps channel-major with streaming stores, forward taps at [0, L), reverse taps
+// mirrored into [L, 2L) (bert/src/mm/hyena_utils.py:175,213-217,233-234).
+template <int TILES, class TAB, bool PROJECT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void hidden_kernel(TAB tab, int L, int emb, float w_mod,
                                                      const uint16_t* __restrict__ wsplit,
                                                      uint16_t* __restrict__ h_hi /* (2 nf, L, 128) bf16 */,
-                                                     uint16_t* __restrict__ h_lo /* (2 nf, L, 128) bf16 */) {
+                                                     uint16_t* __restrict__ h_lo /* (2 nf, L, 128) bf16 */,
+                                                     int d, float shift, const uint16_t* __restrict__ w3split,
+                                                     float* __restrict__ taps /* (nf, d, 2L) */) {
   constexpr int P = 32 * TILES;
   __shared__ __attribute__((aligned(16))) unsigned char act[3][P * kActRowB];
   __shared__ float zt[P * kMaxEmb];
@@ -119,8 +128,14 @@ __global__ __launch_bounds__(256) void hidden_kernel(TAB tab, int L, int emb, fl
   const int fi = blockIdx.y >> 1, dir = blockIdx.y & 1;
   const FilterPtrs& F = tab.at(fi);
   const MlpPtrs& W = F.mlp[dir];
-  if (W.w0 == nullptr) return;                  // not bidirectional: nothing to do for dir == 1
   const int l0 = blockIdx.x * P;
+  if (W.w0 == nullptr) {                        // not bidirectional: nothing to compute for dir == 1 ...
+    if constexpr (PROJECT) {                    // ... and the reverse half of the window is zero
+      float* out = taps + (long)fi * d * 2 * L + (2L * L - l0 - P);
+      for (int i = tid; i < d * P; i += 256) out[(long)(i / P) * 2 * L + i % P] = 0.f;
+    }
+    return;
+  }
 
   auto put3 = [&](int pos, int o, float v0, float v1, float v2, float v3) __attribute__((always_inline)) {
     float h[4], m[4], l[4];
@@ -217,6 +232,16 @@ __global__ __launch_bounds__(256) void hidden_kernel(TAB tab, int L, int emb, fl
       for (int j = 0; j < 4; ++j) s[j] = sin_reduced(fr[4 * vq + j] * (acc[4 * vq + j] + bs[4 * vq + j]));
       if constexpr (layer == 0) {
         put3(pos, o, s[0], s[1], s[2], s[3]);
+      } else if constexpr (PROJECT) {           // h3 = hi + lo stays in LDS (parts 0 and 1) for the projection
+        float hi[4], lo[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          hi[j] = bf16_to_f32(f32_to_bf16(s[j]));
+          lo[j] = s[j] - hi[j];
+        }
+        const int off = pos * kActRowB + 2 * o;
+        *reinterpret_cast<uint2*>(&act[0][off]) = make_uint2(pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3]));
+        *reinterpret_cast<uint2*>(&act[1][off]) = make_uint2(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]));
       } else {
         const long hrow = ((long)blockIdx.y * L + l0 + pos) * kOrder;
         float hi[4], lo[4];
@@ -251,6 +276,71 @@ __global__ __launch_bounds__(256) void hidden_kernel(TAB tab, int L, int emb, fl
   layer_pass(ic<0>{});
   load_scales(1);
   layer_pass(ic<1>{});
+
+  if constexpr (PROJECT) {
+    // the barrier that ended the last layer says h3 (hi in act[0], lo in act[1]) is complete for all P positions
+    float* out = taps + (long)fi * d * 2 * L;
+    const u32x4* w3 = reinterpret_cast<const u32x4*>(w3split + (long)blockIdx.y * 2 * d * kOrder) + lane;
+    float tl[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) tl[t] = F.t[l0 + 32 * t + i32];
+    // A operand of a channel tile: weight rows 32 ct + i32, K = 16 ks + 8 half + {0..7}, hi / lo parts as
+    // split_weights_kernel left them, and the decay rates of the lane's 16 channels
+    struct TileOps {
+      bf16x8 ahi[kOrder / 16], alo[kOrder / 16];
+      float4 dq[4];
+    };
+    auto fetch_tile = [&](int ct, TileOps& o) __attribute__((always_inline)) {
+#pragma unroll
+      for (int ks = 0; ks < kOrder / 16; ++ks) {
+        o.ahi[ks] = __builtin_bit_cast(bf16x8, w3[(ct * 8 + ks) * 64]);
+        o.alo[ks] = __builtin_bit_cast(bf16x8, w3[(ct * 8 + ks) * 64 + d * kOrder / 8]);
+      }
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) o.dq[vq] = *reinterpret_cast<const float4*>(F.deltas + 32 * ct + 8 * vq + 4 * half);
+    };
+    auto project_tile = [&](int ct, const TileOps& o) __attribute__((always_inline)) {
+      float adelta[16];
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) {
+        adelta[4 * vq] = -fabsf(o.dq[vq].x) * 1.44269504088896341f; adelta[4 * vq + 1] = -fabsf(o.dq[vq].y) * 1.44269504088896341f;
+        adelta[4 * vq + 2] = -fabsf(o.dq[vq].z) * 1.44269504088896341f; adelta[4 * vq + 3] = -fabsf(o.dq[vq].w) * 1.44269504088896341f;
+      }
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) {
+        const unsigned char* bh = &act[0][(32 * t + i32) * kActRowB + 16 * half];
+        const unsigned char* bl = &act[1][(32 * t + i32) * kActRowB + 16 * half];
+        floatx16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < kOrder / 16; ++ks) {
+          const bf16x8 bhi = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(bh + 32 * ks));
+          const bf16x8 blo = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(bl + 32 * ks));
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.alo[ks], bhi, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.ahi[ks], blo, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.ahi[ks], bhi, acc, 0, 0, 0);
+        }
+        // accumulator element v of lane: channel 32 ct + 8 (v / 4) + 4 half + v % 4, position l0 + 32 t + i32
+        const int l = l0 + 32 * t + i32;
+        float* po = out + (long)(32 * ct + 4 * half) * 2 * L + (dir == 0 ? l : (2L * L - 1 - l));
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          // exp(-t |delta|); the bare hardware exp2 flushes results below 2^-126 to zero, which is the value to
+          // 1e-38 absolute.  Streaming store: the taps are read once, by a later kernel
+          const float decay = __builtin_amdgcn_exp2f(tl[t] * adelta[v]) + shift;
+          __builtin_nontemporal_store(acc[v] * decay, po + (long)(8 * (v >> 2) + (v & 3)) * 2 * L);
+        }
+      }
+    };
+    // (a second register set that requests the next tile's operands ahead was measured: the registers it needs
+    // beside the hidden layers' spill, 120 against 82 us per mixer at L = 8192)
+    TileOps o;
+    for (int ct = w; ct < d / 32; ct += 4) {
+      fetch_tile(ct, o);
+      project_tile(ct, o);
+    }
+  }
 }
 
 // Workgroup = 4 waves = 128 channels; wave w owns channels [c0 + 32 w, + 32) with its weight rows split
@@ -259,7 +349,7 @@ __global__ __launch_bounds__(256) void hidden_kernel(TAB tab, int L, int emb, fl
 // LDS (double buffered, rows padded to 272 bytes so that the 16-byte operand reads of 32 rows spread over
 // all banks) and shared by the four waves.
 // grid (L / kPosPerWg rounded up, d / 128 rounded up, 2 * nfilters).
-constexpr int kPosPerWg = 256;      // at most; 32-position tiles past L are skipped
+constexpr int kPosPerWg = 512;      // at most; 32-position tiles past L are skipped
 constexpr int kHRow = 2 * kOrder + 16;   // bytes per padded LDS row of one h3 part
 template <class TAB>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) void project_kernel(TAB tab, int L, int d, float shift,
@@ -353,7 +443,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
         // exp(-t |delta|); the bare hardware exp2 flushes results below 2^-126 to zero, which is the
         // value to 1e-38 absolute
         const float decay = __builtin_amdgcn_exp2f(tl * adelta[v]) + shift;
-        po[(long)(8 * (v >> 2) + (v & 3)) * 2 * L] = acc[v] * decay;
+        // streaming store: the taps (100 MB per mixer at L = 8192) are read once, by a later kernel (-5 % for the call)
+        __builtin_nontemporal_store(acc[v] * decay, po + (long)(8 * (v >> 2) + (v & 3)) * 2 * L);
       }
     }
     if (pt + 1 < ntiles) stage(P ^ 1, ic<P ^ 1>{});
@@ -390,10 +481,18 @@ static int filter_launches(TAB tab, int nfilters, int L, int d, int emb_dim, flo
   if (rc) return rc;
   // positions per workgroup: longer runs amortise the weight fetch (96 KB per workgroup and layer), short sequences
   // need the workgroups spread over the chip
-  if (L % 64 == 0 && L >= 1024)      // measured at L = 8192: 26.9 us with two tiles, 29.5 with four, 32.7 with one
-    hipLaunchKernelGGL((hidden_kernel<2, TAB>), dim3(L / 64, 2 * nfilters), dim3(256), 0, s, tab, L, emb_dim, w_mod, wsplit, h_hi, h_lo);
-  else
-    hipLaunchKernelGGL((hidden_kernel<1, TAB>), dim3(L / 32, 2 * nfilters), dim3(256), 0, s, tab, L, emb_dim, w_mod, wsplit, h_hi, h_lo);
+  if (L % 64 == 0 && L >= 1024) {     // measured at L = 8192: 26.9 us with two tiles, 29.5 with four, 32.7 with one
+    if (taps && d % 32 == 0) {        // hidden layers and projection as one kernel: h3 never leaves the chip
+      hipLaunchKernelGGL((hidden_kernel<2, TAB, true>), dim3(L / 64, 2 * nfilters), dim3(256), 0, s, tab, L, emb_dim, w_mod, wsplit,
+                         h_hi, h_lo, d, shift, w3split, taps);
+      return check_launch("hyena hidden + project kernel");
+    }
+    hipLaunchKernelGGL((hidden_kernel<2, TAB, false>), dim3(L / 64, 2 * nfilters), dim3(256), 0, s, tab, L, emb_dim, w_mod, wsplit,
+                       h_hi, h_lo, 0, 0.f, nullptr, nullptr);
+  } else {
+    hipLaunchKernelGGL((hidden_kernel<1, TAB, false>), dim3(L / 32, 2 * nfilters), dim3(256), 0, s, tab, L, emb_dim, w_mod, wsplit,
+                       h_hi, h_lo, 0, 0.f, nullptr, nullptr);
+  }
   rc = check_launch("hyena hidden_kernel");
   if (rc || !taps) return rc;
   hipLaunchKernelGGL(project_kernel<TAB>, dim3((L + kPosPerWg - 1) / kPosPerWg, (d + 127) / 128, 2 * nfilters), dim3(256), 0, s, tab, L, d, shift,
