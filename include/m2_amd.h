@@ -79,9 +79,9 @@ int m2_hyena_filter_fwd(const m2_hyena_filter_params* params, int nfilters, int 
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The intermediate activations
  * go through a device array of M2_HYENA_FILTER_STATIC_SCRATCH_BYTES that is part of the library itself (every GPU
  * the library runs on holds one copy until the process ends); the call allocates and frees nothing.  Limit:
- * m2_hyena_filter_workspace_bytes(nfilters, L, d, order) must not exceed that size: 20 MiB holds nfilters * L <= 16384
- * for every d <= 1536 (both filters of a mixer up to L = 8192 at d = 768 need 19,136,512 bytes, at d = 1536
- * 20,709,376); beyond it the call fails with M2_ERR_UNSUPPORTED.  All calls on one GPU share
+ * m2_hyena_filter_workspace_bytes(nfilters, L, d, order) must not exceed that size: 20 MiB holds both filters of a
+ * mixer up to L = 8192, or one filter up to L = 16384, for every d <= 1536 (two filters at L = 8192 need 19,136,512
+ * bytes at d = 768 and 20,709,376 at d = 1536); beyond it the call fails with M2_ERR_UNSUPPORTED.  All calls on one GPU share
  * the array: two such calls whose kernels may overlap on the same GPU (different streams, or different host threads
  * on different streams) race; calls on one stream are ordered and safe.  The first call on a device looks up the
  * array's device address (hipGetSymbolAddress): make that call outside a stream capture. */
@@ -152,16 +152,6 @@ int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, const float* u,
  * of `spec` (HyenaFilter.forward on its own, bert/src/mm/hyena_utils.py:219-248).
  * x, y (d, B, L) channel-major, act_dtype. */
 int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, int L, int d, int act_dtype, void* stream);
-
-/* ---------------------------------------------------------------------------------------------
- * Dense projection of the sequence mixer (in_linear, bert/src/mm/monarch_mixer_sequence_mixer.py:81,108) written
- * straight into the channel-major layout m2_mixer_core_fwd reads:
- *   out[q][p] = sum_k Q[q][k] P[p][k],   P (np, K), Q (nq, K), out (nq, np), all bf16, dense, fp32 accumulation.
- * With P = the layer input (M, d) and Q = in_linear.weight (3d, d) the result is xproj (3d, M); the bias is left
- * to m2_mixer_core_fwd (proj_bias).  The reference runs this as nn.Linear followed by a transpose.
- * Needs K % 64 == 0 and operands below 4 GiB each. */
-int m2_gemm_bf16_supported(int np, int nq, int K);
-int m2_gemm_bf16_qmajor_fwd(const void* P, const void* Q, void* out, int np, int nq, int K, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Block-diagonal ("Monarch") linear layers of the GLU MLP, bf16 MFMA with fp32 accumulation.

@@ -57,10 +57,6 @@ def _load() -> ctypes.CDLL:
     lib.m2_mixer_filters_fwd.restype = c_int
     lib.m2_mixer_filters_fwd.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float,
                                          c_void_p, c_void_p, c_void_p]
-    lib.m2_gemm_bf16_supported.restype = c_int
-    lib.m2_gemm_bf16_supported.argtypes = [c_int, c_int, c_int]
-    lib.m2_gemm_bf16_qmajor_fwd.restype = c_int
-    lib.m2_gemm_bf16_qmajor_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]
     lib.m2_blockdiag_glu_fwd.restype = c_int
     lib.m2_blockdiag_glu_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
     lib.m2_blockdiag_linear_fwd.restype = c_int
@@ -104,7 +100,7 @@ lib = _load()
 
 EXPORTS = ["m2_version", "m2_last_error", "m2_hyena_filter_workspace_bytes", "m2_hyena_filter_fwd", "m2_hyena_filter_fwd_static", "m2_mixer_filters_workspace_bytes", "m2_mixer_filters_fwd",
            "m2_fftconv_supported_seqlen", "m2_filter_spectrum_bytes", "m2_filter_spectrum_fwd", "m2_mixer_core_fwd",
-           "m2_fftconv_fwd", "m2_gemm_bf16_supported", "m2_gemm_bf16_qmajor_fwd", "m2_blockdiag_glu_fwd", "m2_blockdiag_linear_fwd", "m2_blockdiag_linear_f32_fwd", "m2_mlp_fused_supported", "m2_mlp_fused_packed_bytes", "m2_mlp_fused_pack", "m2_mlp_fused_fwd", "m2_glu_stream_supported", "m2_glu_stream_packed_bytes", "m2_glu_stream_pack", "m2_glu_stream_fwd", "m2_layernorm_fwd", "m2_layernorm_bf16_fwd",
+           "m2_fftconv_fwd", "m2_blockdiag_glu_fwd", "m2_blockdiag_linear_fwd", "m2_blockdiag_linear_f32_fwd", "m2_mlp_fused_supported", "m2_mlp_fused_packed_bytes", "m2_mlp_fused_pack", "m2_mlp_fused_fwd", "m2_glu_stream_supported", "m2_glu_stream_packed_bytes", "m2_glu_stream_pack", "m2_glu_stream_fwd", "m2_layernorm_fwd", "m2_layernorm_bf16_fwd",
            "m2_embed_layernorm_fwd", "m2_blockdiag_linear_layernorm_supported", "m2_blockdiag_linear_layernorm_fwd"]
 
 

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libm2_amd.so")
 SOURCES = ["common.hip", "fftconv_kernels.hip", "fftconv_real_kernels.hip", "fftconv_split_kernels.hip", "hyena_filter_kernels.hip", "filter_fused_kernels.hip", "blockdiag_kernels.hip", "wo_layernorm_kernels.hip",
-           "mlp_fused_kernels.hip", "glu_stream_kernels.hip", "gemm_kernels.hip"]
+           "mlp_fused_kernels.hip", "glu_stream_kernels.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 VALU instructions are switched off on purpose (device flag, the host pass warns about it)
 FLAGS = ["-std=c++17", "-O3", "--offload-arch=gfx950", "-fPIC", "-Xclang", "-target-feature", "-Xclang",

@@ -10,16 +10,17 @@
 
 namespace m2 {
 
-// LDS padding of the row buffer: two slots after every 32 and one more after every 512.  With it the staging
-// layout (32 consecutive slots per thread), the first pass (consecutive threads, consecutive slots at stride
-// L / R1) and the second pass (16 consecutive slots per 256) are all free of bank conflicts for 8-byte
-// accesses (checked by enumerating the 64 banks for every access pattern of the L = 8192 plan).
-__device__ __forceinline__ int sphys(int pos) { return pos + 2 * (pos >> 5) + (pos >> 9); }
+// LDS padding of the row buffer: one slot after every 16 and one more after every 256.  Chosen by measurement among
+// the paddings whose offsets stay linear for every access pattern (split_offsets_ok below): at L = 8192 the
+// bank-conflict counter of the mixer kernel reads 2.6 M cycles per launch with it against 9.4 M for two slots after
+// every 32 plus one after every 512 (which a 64-bank model of 8-byte accesses rates conflict-free), 5.5 M for
+// (16, 512) and 35 M for one slot after every 8; the kernel is 2 - 3 % faster.
+__host__ __device__ constexpr int sphys(int pos) { return pos + (pos >> 4) + (pos >> 8); }
 // Padded offset of logical offset `o` relative to a base position: valid where adding `o` to the base carries
-// neither into bit 5 nor into bit 9 from below (every access in this file: offsets are multiples of 256 on a
-// base below 256, multiples of 16 below 256 on a base whose low byte is below 16, or below 16 / 32 on a base
-// that is a multiple of 16 / 32).
-constexpr int spoff(int o) { return o + 2 * (o >> 5) + (o >> 9); }
+// neither into bit 4 nor into bit 8 from below (every access in this file: offsets are multiples of 256 on a
+// base below 256, multiples of 16 below 256 on a base whose low byte is below 16, or below 16 on a base
+// that is a multiple of 16).
+constexpr int spoff(int o) { return o + (o >> 4) + (o >> 8); }
 
 template <int LOGL_, int R1_, int R2_>
 struct SplitPlan {
@@ -30,13 +31,30 @@ struct SplitPlan {
   static constexpr int M = L / RP;                // groups of 16 in the last pass
   static constexpr int S1 = L / R1, S2 = S1 / R2;
   static constexpr int NB1 = E / R1, NB2 = E / R2;
-  static constexpr int ROW_LDS = L + 2 * (L >> 5) + (L >> 9);    // padded complex slots of the row buffer
+  static constexpr int ROW_LDS = L + (L >> 4) + (L >> 8);    // padded complex slots of the row buffer
   static constexpr int TAB2 = R2 * S2;            // pass-2 twiddle table
   static constexpr int WG_LDS = ROW_LDS + TAB2;   // float2 slots per workgroup
   static_assert(R1 * R2 * RP == L, "radices must multiply to L");
   static_assert(S2 == RP, "last stride");
   static_assert(R1 % 8 == 0 && R1 <= 32 && R2 <= 32, "radix range");
 };
+
+// sphys(base + o) == sphys(base) + spoff(o) for every (base, offset) pair the passes of plan P use
+template <class P>
+constexpr bool split_offsets_ok() {
+  for (int q = 0; q < P::S1; ++q)
+    for (int j = 0; j < P::R1; ++j)
+      if (sphys(q + j * P::S1) != sphys(q) + spoff(j * P::S1)) return false;
+  for (int q = 0; q < P::L / P::R2; ++q) {
+    const int base = (q / P::S2) * (P::S2 * P::R2) + q % P::S2;
+    for (int j = 0; j < P::R2; ++j)
+      if (sphys(base + j * P::S2) != sphys(base) + spoff(j * P::S2)) return false;
+  }
+  for (int g = 0; g < P::M; ++g)
+    for (int j = 0; j < 16; ++j)
+      if (sphys(16 * g + j) != sphys(16 * g) + j) return false;
+  return sphys(P::L - 1) < P::ROW_LDS;
+}
 
 // cos of 2 pi k / 64 for k = 0 .. 16
 constexpr float kCos64[17] = {1.0f,

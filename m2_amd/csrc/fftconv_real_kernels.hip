@@ -461,6 +461,7 @@ __global__ __launch_bounds__(P::T) void filter_spectrum_real_kernel(
 // host-side launchers
 // ------------------------------------------------------------------------------------------
 typedef SplitPlan<14, 32, 32> RealPlan;      // half transforms of 16384 points: sequence length 32768
+static_assert(split_offsets_ok<RealPlan>(), "LDS offsets of the split plan");
 
 size_t real_spectrum_bytes(int d) { return (size_t)d * 4 * real_spec_block<RealPlan>() * sizeof(float); }
 

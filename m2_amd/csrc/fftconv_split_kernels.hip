@@ -369,6 +369,10 @@ static int launch_filter_spectrum_split_t(const float* taps1, const float* taps2
   X(13, 32, 16)                   \
   X(14, 32, 32)
 
+#define X(LOGL, R1, R2) static_assert(split_offsets_ok<SplitPlan<LOGL, R1, R2>>(), "LDS offsets of the split plan");
+M2_FOR_EACH_SPLIT_PLAN(X)
+#undef X
+
 bool split_plan_exists(int L) {
   switch (L) {
 #define X(LOGL, R1, R2) \

@@ -254,10 +254,7 @@ class BertLayer(nn.Module):
         # output: the same product as W @ h16^T, for which the library picks a faster kernel (126 against 144 us at
         # M = 32768, d = 768)
         xproj = torch.empty(3 * d, B * L, dtype=torch.bfloat16, device=h16.device)
-        if at.own_in_linear:
-            ops.gemm_qmajor(h16, w_in, out=xproj)
-        else:
-            torch.mm(h16, w_in.t(), out=xproj.t())
+        torch.mm(h16, w_in.t(), out=xproj.t())
         if spec_ready is not None:
             torch.cuda.current_stream().wait_event(spec_ready)
         y = at.core(xproj.view(3 * d, B, L), hT.view(d, B, L) if at.residual_long_conv else None, B, L, spec=spec)

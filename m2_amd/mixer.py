@@ -58,10 +58,6 @@ class MonarchMixerSequenceMixing(nn.Module):
         self.short_filter = nn.Conv1d(in_channels=total_width, out_channels=total_width, kernel_size=3,
                                       groups=total_width, padding=2)
         self._cast_cache = {}
-        # True: the in-projection of the fused encoder schedule runs on this library's own MFMA kernel
-        # (m2_gemm_bf16_qmajor_fwd) instead of the library GEMM.  Off by default: measured on MI355X the library is
-        # faster (843 against 655 TFLOP/s at M = 32768, d = 768; 1214 against 647 at M = 8192, d = 1536).
-        self.own_in_linear = False
         self.cache_filters = False
         self._spec_cache = None
         self._filter_table = None

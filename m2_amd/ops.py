@@ -59,7 +59,7 @@ def hyena_filter_taps(filters: Sequence[dict], L: int, d: int, order: int, emb_d
     Each entry is a dict with fp32 GPU tensors: z (>=L, emb), t (>=L), freq (order), deltas (d),
     `fwd` = [w0, b0, w1, b1, w2, b2, w3] and optionally `rev` = the same seven of the reverse MLP.
     `static_scratch=True` takes the library's allocation-free entry point (m2_hyena_filter_fwd_static: no
-    workspace tensor; the 20 MiB static array holds nfilters * L <= 16384 for d <= 1536); with `out` given as well
+    workspace tensor; the 20 MiB static array holds two filters up to L = 8192 or one up to L = 16384 for d <= 1536); with `out` given as well
     nothing is allocated at all.
     """
     nf = len(filters)
@@ -227,23 +227,6 @@ def fftconv(x: Tensor, spec: Tensor, B: int, L: int, d: int) -> Tensor:
     _require(spec, "spec", torch.float32, (lib.m2_filter_spectrum_bytes(d, L) // 4,))
     out = torch.empty_like(x)
     check(lib.m2_fftconv_fwd(_ptr(x), _ptr(spec), _ptr(out), B, L, d, code, _stream()))
-    return out
-
-
-def gemm_qmajor(P: Tensor, Q: Tensor, out: Optional[Tensor] = None) -> Tensor:
-    """out (nq, np) = Q @ P^T for P (np, K), Q (nq, K) bf16 (fp32 accumulation): with P the tokens (M, d) and Q a
-    weight (n, d) this is the projection written channel-major (n, M)."""
-    np_, K = P.shape
-    nq, K2 = Q.shape
-    _require(P, "P", torch.bfloat16)
-    _require(Q, "Q", torch.bfloat16)
-    if K != K2:
-        raise ValueError(f"P has K = {K}, Q has K = {K2}")
-    if out is None:
-        out = torch.empty(nq, np_, dtype=torch.bfloat16, device=P.device)
-    else:
-        _require(out, "out", torch.bfloat16, (nq, np_))
-    check(lib.m2_gemm_bf16_qmajor_fwd(_ptr(P), _ptr(Q), _ptr(out), np_, nq, K, _stream()))
     return out
 
 

@@ -286,13 +286,11 @@ def test_encoder_small(gpu, L, B, layers):
     out1, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
     e, e2 = rel_err(out1, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
-    # the MLP as two kernels with an fp32 sum into the LayerNorm (the default is one kernel and a bf16 sum), and the
-    # in-projection on this library's own GEMM kernel
+    # the MLP as two kernels with an fp32 sum into the LayerNorm (the default is one kernel and a bf16 sum)
     for layer in model.encoder.layer:
         layer.mlp.fuse_wo_layernorm = False
         layer.mlp.fuse_mlp = False
         layer.mlp.bf16_presum = False
-        layer.attention.own_in_linear = True
     out2, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
     e, e2 = rel_err(out2, ref)
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
@@ -729,24 +727,6 @@ def test_mlp_fused_matches_oracle_and_the_two_kernel_path(gpu, M, I):
         ops.mlp_fused(torch.zeros(8, 512, device=gpu, dtype=torch.bfloat16),
                       torch.zeros(4, 256, 128, device=gpu, dtype=torch.bfloat16),
                       torch.zeros(4, 128, 128, device=gpu, dtype=torch.bfloat16))
-
-
-@pytest.mark.parametrize("np_,nq,K", [(256, 256, 64), (4096, 2304, 768), (1000, 300, 128), (32768, 2304, 768),
-                                     (8192, 4608, 1536), (257, 513, 192)])
-def test_gemm_qmajor_projection(gpu, np_, nq, K):
-    """The dense projection kernel (in_linear written channel-major) against fp64 on the bf16 operands, ragged
-    tiles both ways."""
-    from m2_amd import ops
-    g = torch.Generator().manual_seed(np_ + nq)
-    P = torch.randn(np_, K, generator=g).bfloat16()
-    Q = (torch.randn(nq, K, generator=g) * 0.05).bfloat16()
-    got = ops.gemm_qmajor(P.to(gpu), Q.to(gpu))
-    assert got.shape == (nq, np_) and got.dtype == torch.bfloat16
-    ref = (Q.float() @ P.float().T).double() if np_ * nq > 4e6 else Q.double() @ P.double().T
-    e, e2 = rel_err(got.float(), ref)
-    assert e < TOL_BF16 and e2 < 4e-3, (e, e2)
-    with pytest.raises(RuntimeError, match="multiple of 64"):
-        ops.gemm_qmajor(torch.zeros(8, 100, device=gpu, dtype=torch.bfloat16), torch.zeros(8, 100, device=gpu, dtype=torch.bfloat16))
 
 
 @pytest.mark.parametrize("M,in_f,out_f,nb", [(300, 768, 6144, 4), (65, 256, 100, 4), (1, 64, 8, 2), (1000, 3072, 768, 4)])
