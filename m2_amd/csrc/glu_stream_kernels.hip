@@ -239,6 +239,7 @@ extern "C" int m2_glu_stream_fwd(const void* x, const void* w_packed, void* out,
   const int ntiles = (M + kSRows - 1) / kSRows;
   // one persistent workgroup per compute unit (144 KB of LDS each), an even number per XCD
   int per_xcd = (num_cus() / 8) & ~1;
+  if (per_xcd < 2) per_xcd = 2;      // a device (or partition) with fewer than 16 compute units: work is dealt to 8 x per_xcd slots whatever the real count
   if (per_xcd > 2 * ((ntiles + 3) / 4)) per_xcd = 2 * ((ntiles + 3) / 4);
   auto kern = glu_stream_kernel;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kSLds);

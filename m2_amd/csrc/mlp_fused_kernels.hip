@@ -410,6 +410,7 @@ extern "C" int m2_mlp_fused_fwd(const void* x, const void* w_packed, const float
   const int ntiles = (M + rows - 1) / rows;
   // one persistent workgroup per compute unit (144 KB of LDS each), an even number per XCD
   int per_xcd = (num_cus() / 8) & ~1;
+  if (per_xcd < 2) per_xcd = 2;      // a device (or partition) with fewer than 16 compute units: work is dealt to 8 x per_xcd slots whatever the real count
   if (per_xcd > 2 * ((ntiles + 3) / 4)) per_xcd = 2 * ((ntiles + 3) / 4);
   const dim3 grid(8 * per_xcd);
   hipStream_t st = (hipStream_t)stream;
