@@ -695,6 +695,18 @@ def test_bench_prints_its_json_line(gpu, extra):
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
 
 
+def test_bench_reference_benchmark_form(gpu):
+    """bench.py --reference-benchmark (random hidden states into the encoder, masked-LM head on top: the form of
+    bert/benchmark_fwd.py:38-80) at the shortest length of the reference's grid: one JSON line, tokens per ms."""
+    import json, os, subprocess, sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "2", "--warmup", "1", "--config", "l512",
+                        "--reference-benchmark"], capture_output=True, text=True, timeout=110, cwd=root)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = json.loads(r.stdout.strip().splitlines()[-1])
+    assert line["unit"] == "tokens/ms" and line["value"] > 0, line
+
+
 @pytest.mark.parametrize("M,I", [(1, 3072), (100, 3072), (128, 3072), (300, 1536), (4096, 3072), (32768 - 70, 3072),
                                  (130, 256)])
 def test_mlp_fused_matches_oracle_and_the_two_kernel_path(gpu, M, I):
