@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Throughput of the M2-BERT-80M encoder forward on one MI355X, sequences per second.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--reps R] [--config c3|c2|c4|c5|l512|l1024|l2048|l4096]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--reps R] [--config c3|c2|c4|c5|l512|l1024|l2048|l4096|m110|m341]
                     [--no-cpu-baseline] [--eager]
 
 A step is one forward of embeddings + 12 Monarch-Mixer layers over one synthetic batch that is
@@ -103,6 +103,14 @@ def workload(name: str):
         cfg, B, pad = m2_amd.m2_bert_large(128, 24), 64, False
         label = "M2-BERT large 24x1536 encoder fwd, L=128, B=64 (config 4)"
         idx = 4
+    elif name == "m110":
+        cfg, B, pad = m2_amd.m2_bert_110m(2048), 16, False
+        label = "M2-BERT 12x960 encoder fwd, L=2048, B=16 (the reference's 960-wide model: 240-wide MLP blocks)"
+        idx = 5
+    elif name == "m341":
+        cfg, B, pad = m2_amd.m2_bert_341m(2048), 16, False
+        label = "M2-BERT 12x1792 encoder fwd, L=2048, B=16 (the reference's 1792-wide model)"
+        idx = 6
     elif name in REFERENCE_GRID:
         Lg, B = REFERENCE_GRID[name]
         cfg, pad = m2_amd.m2_bert_80m(Lg), False

@@ -162,15 +162,16 @@ int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, int L, int 
 
 /* out[m, j] = gelu_erf(h[m, j]) * h[m, I + j],  h = blockdiag_multiply(x, w),  j < I = intermediate.
  * x (M, in_features) bf16 row-major; w (nblocks, 2I/nblocks, in_features/nblocks) bf16 (the
- * `gated_layers.weight` tensor); out (M, I) bf16.  Needs nblocks even, (in/nblocks) % 64 == 0,
- * (2I/nblocks) % 64 == 0. */
+ * `gated_layers.weight` tensor); out (M, I) bf16.  Needs nblocks even, (in/nblocks) % 8 == 0,
+ * (2I/nblocks) % 8 == 0 (block sizes off the kernels' 64-wide tile grid, such as the 240-wide blocks of the
+ * reference's 960-wide model, run on a masked variant of the general kernel). */
 int m2_blockdiag_glu_fwd(const void* x, const void* w, void* out, int M, int in_features, int intermediate,
                          int nblocks, void* stream);
 
 /* out = blockdiag_multiply(x, w) (+ bias) (+ residual).
  * x (M, in_features) bf16; w (nblocks, out/nblocks, in/nblocks) bf16; bias (out_features) fp32 or NULL;
  * residual (M, out_features) bf16 or NULL; out (M, out_features) of out_dtype (M2_DTYPE_F32 / _BF16).
- * Needs (in/nblocks) % 64 == 0, (out/nblocks) % 64 == 0. */
+ * Needs (in/nblocks) % 8 == 0, (out/nblocks) % 8 == 0. */
 int m2_blockdiag_linear_fwd(const void* x, const void* w, const float* bias, const void* residual, void* out, int M,
                             int in_features, int out_features, int nblocks, int out_dtype, void* stream);
 

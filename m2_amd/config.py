@@ -65,3 +65,15 @@ def m2_bert_large(seq_len: int = 128, num_hidden_layers: int = 24) -> M2BertConf
     """d_model 1536 / intermediate 6144 (bert/yamls/pretrain/monarch-mixer-large-pretrain-1536dim-260m-parameters.yaml)."""
     return replace(M2BertConfig(), hidden_size=1536, intermediate_size=6144, num_hidden_layers=num_hidden_layers,
                    num_attention_heads=24).with_seq_len(seq_len)
+
+
+def m2_bert_110m(seq_len: int = 128) -> M2BertConfig:
+    """d_model 960 / intermediate 3840, 12 layers: the parameter-matched model
+    (bert/yamls/pretrain/monarch-mixer-pretrain-960dim-parameter-matched.yaml:17-24).  Its MLP blocks are 240 wide."""
+    return replace(M2BertConfig(), hidden_size=960, intermediate_size=3840).with_seq_len(seq_len)
+
+
+def m2_bert_341m(seq_len: int = 128) -> M2BertConfig:
+    """d_model 1792 / intermediate 7168, 12 layers
+    (bert/yamls/pretrain/monarch-mixer-large-pretrain-1792dim-341m-parameters.yaml:17-24)."""
+    return replace(M2BertConfig(), hidden_size=1792, intermediate_size=7168).with_seq_len(seq_len)

@@ -63,7 +63,10 @@ __device__ __forceinline__ float gelu_erf(float x) {
 constexpr int kBK = 64;
 constexpr int kLdsRow = kBK + 8;          // bf16 elements per padded LDS row (144 bytes)
 
-template <int WR, int WC, bool GLU, typename OUT, int NSTAGE>
+// RAG: block sizes that are not multiples of the tile (p, q multiples of 8 only, e.g. the 240-wide blocks of
+// d = 960): the last K chunk of a block is filled with zeros beyond p, the last column tile of a block computes
+// on clamped weight rows and stores only the columns below q.
+template <int WR, int WC, bool GLU, typename OUT, int NSTAGE, bool RAG = false>
 __global__ __launch_bounds__(64 * WR * WC) void blockdiag_kernel(
     const uint16_t* __restrict__ x,      // (M, nb p) bf16
     const uint16_t* __restrict__ w,      // (nb, q, p) bf16
@@ -83,7 +86,7 @@ __global__ __launch_bounds__(64 * WR * WC) void blockdiag_kernel(
   // weights of the tiles in flight on an XCD stay in that XCD's L2.
   int tile_m, tile_n;
   {
-    const int ntm = (M + BM - 1) / BM, ntn = (GLU ? nb * q / 2 : nb * q) / BN;
+    const int ntm = (M + BM - 1) / BM, ntn = (GLU ? nb / 2 : nb) * ((q + BN - 1) / BN);
     const int id = blockIdx.x, e = id & 7, l = id >> 3;
     const int full = (ntm / 8) * 8;                   // row tiles covered by the XCD-striped part
     if (id < full * ntn) {
@@ -96,11 +99,13 @@ __global__ __launch_bounds__(64 * WR * WC) void blockdiag_kernel(
     }
   }
   const int m0 = tile_m * BM;
-  const int n0 = tile_n * BN;                         // first output column of the tile
+  const int ntn_b = (q + BN - 1) / BN;                // column tiles per block
+  const int blk = tile_n / ntn_b, jj = (tile_n % ntn_b) * BN;      // weight block and first row inside it (gate block for GLU)
+  const int n0 = blk * q + jj;                        // first output column of the tile
   const int in_f = nb * p;
-  const int blk = n0 / q, jj = n0 % q;                // weight block and first row inside it (gate block for GLU)
   const int out_cols = GLU ? nb * q / 2 : nb * q;
-  const int kchunks = p / kBK;
+  const int kchunks = (p + kBK - 1) / kBK;
+  const int kc8 = (tid & 7) * 8;                      // K offset of every 16-byte piece this thread moves (NT is a multiple of 8)
   const int nchunks = GLU ? 2 * kchunks : kchunks;
 
   // per-thread source rows of the 16-byte chunks it moves (fixed for the whole kernel)
@@ -118,7 +123,9 @@ __global__ __launch_bounds__(64 * WR * WC) void blockdiag_kernel(
   static_for<0, B_CH>([&](auto jj_) {
     constexpr int j = decltype(jj_)::value;
     const int id = tid + NT * j, r = id >> 3, kc = id & 7;
-    pb[j] = w + ((long)blk * q + jj + r) * p + kc * 8;
+    int wrow = jj + r;
+    if constexpr (RAG) wrow = wrow < q ? wrow : q - 1;      // columns past the block's end: computed, never stored
+    pb[j] = w + ((long)blk * q + wrow) * p + kc * 8;
     lb[j] = (BM + r) * kLdsRow + kc * 8;
   });
   const long a_phase = (long)(nb / 2) * p;            // value block = gate block + nb/2
@@ -129,6 +136,14 @@ __global__ __launch_bounds__(64 * WR * WC) void blockdiag_kernel(
     const int phase = GLU ? c / kchunks : 0;
     const long ao = phase * a_phase + (c % kchunks) * kBK;
     const long bo = phase * b_phase + (c % kchunks) * kBK;
+    if constexpr (RAG) {
+      if ((c % kchunks) * kBK + kc8 >= p) {           // beyond the block's K range: zeros on both sides
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        static_for<0, A_CH>([&](auto jj_) { ra[decltype(jj_)::value] = z; });
+        static_for<0, B_CH>([&](auto jj_) { rb[decltype(jj_)::value] = z; });
+        return;
+      }
+    }
     static_for<0, A_CH>([&](auto jj_) { ra[decltype(jj_)::value] = *reinterpret_cast<const u32x4*>(pa[decltype(jj_)::value] + ao); });
     static_for<0, B_CH>([&](auto jj_) { rb[decltype(jj_)::value] = *reinterpret_cast<const u32x4*>(pb[decltype(jj_)::value] + bo); });
   };
@@ -187,8 +202,9 @@ __global__ __launch_bounds__(64 * WR * WC) void blockdiag_kernel(
   constexpr int EROWS = BM / EP;
   constexpr int TPR = BN / 4, RPI = NT / TPR;           // each thread moves 4 consecutive columns
   const int cq = (tid % TPR) * 4;
+  const bool col_ok = !RAG || jj + cq < q;             // q is a multiple of 8: four columns are all in or all out
   float4 bq = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (!GLU && bias) bq = *reinterpret_cast<const float4*>(bias + n0 + cq);
+  if (!GLU && bias && col_ok) bq = *reinterpret_cast<const float4*>(bias + n0 + cq);
   for (int ep = 0; ep < EP; ++ep) {
     if (wr / (WR / EP) == ep) {
       float* so = reinterpret_cast<float*>(smem) + ((wr % (WR / EP)) * 64 + 4 * half) * OROW + wc * 64 + i32;
@@ -212,7 +228,7 @@ __global__ __launch_bounds__(64 * WR * WC) void blockdiag_kernel(
         constexpr int i = decltype(ii)::value;
         const int row = m0 + ep * EROWS + tid / TPR + i * RPI;
         rres[i] = make_uint2(0u, 0u);
-        if (resid && row < M) rres[i] = *reinterpret_cast<const uint2*>(resid + (long)row * out_cols + n0 + cq);
+        if (resid && row < M && col_ok) rres[i] = *reinterpret_cast<const uint2*>(resid + (long)row * out_cols + n0 + cq);
       });
     }
     __syncthreads();
@@ -221,7 +237,7 @@ __global__ __launch_bounds__(64 * WR * WC) void blockdiag_kernel(
       constexpr int i = decltype(ii)::value;
       const int r = tid / TPR + i * RPI;
       const int row = m0 + ep * EROWS + r;
-      if (row < M) {
+      if (row < M && col_ok) {
         float4 v4 = *reinterpret_cast<const float4*>(srow + r * OROW);
         const long o = (long)row * out_cols + n0 + cq;
         if constexpr (!GLU) {
@@ -242,19 +258,19 @@ __global__ __launch_bounds__(64 * WR * WC) void blockdiag_kernel(
   }
 }
 
-template <int WR, int WC, bool GLU, typename OUT, int NSTAGE>
+template <int WR, int WC, bool GLU, typename OUT, int NSTAGE, bool RAG = false>
 static int launch_blockdiag(const void* x, const void* w, const float* bias, const void* resid, void* out, int M,
                             int nb, int p, int q, int out_cols, hipStream_t stream) {
   constexpr int BM = 64 * WR, BN = 64 * WC;
   size_t lds = (size_t)NSTAGE * (BM + BN) * kLdsRow * sizeof(uint16_t);
   const size_t epi = (size_t)(BM / (WR == 4 ? 2 : 1)) * (BN + 4) * sizeof(float);
   if (epi > lds) lds = epi;
-  auto kern = blockdiag_kernel<WR, WC, GLU, OUT, NSTAGE>;
+  auto kern = blockdiag_kernel<WR, WC, GLU, OUT, NSTAGE, RAG>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(blockdiag): %s", hipGetErrorString(e));
   }
-  dim3 grid(((M + BM - 1) / BM) * (out_cols / BN));
+  dim3 grid(((M + BM - 1) / BM) * ((out_cols / q) * ((q + BN - 1) / BN)));
   hipLaunchKernelGGL(kern, grid, dim3(64 * WR * WC), lds, stream, (const uint16_t*)x, (const uint16_t*)w, bias,
                      (const uint16_t*)resid, (OUT*)out, M, nb, p, q);
   return check_launch("blockdiag");
@@ -946,8 +962,8 @@ using namespace m2;
 
 static int check_blockdiag(const char* who, int M, int nb, int p, int q, bool glu) {
   if (M <= 0 || nb <= 0 || p <= 0 || q <= 0) return set_error(M2_ERR_ARG, "%s: sizes must be positive (M=%d nb=%d p=%d q=%d)", who, M, nb, p, q);
-  if (p % 64 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: in_features/nblocks=%d must be a multiple of 64", who, p);
-  if (q % 64 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: out_features/nblocks=%d must be a multiple of 64", who, q);
+  if (p % 8 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: in_features/nblocks=%d must be a multiple of 8", who, p);
+  if (q % 8 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: out_features/nblocks=%d must be a multiple of 8", who, q);
   if (glu && nb % 2 != 0) return set_error(M2_ERR_UNSUPPORTED, "%s: GLU pairing needs an even number of blocks, got %d", who, nb);
   return M2_OK;
 }
@@ -961,6 +977,11 @@ extern "C" int m2_blockdiag_glu_fwd(const void* x, const void* w, void* out, int
   const int p = in_features / nblocks, q = 2 * intermediate / nblocks;
   int rc = check_blockdiag("m2_blockdiag_glu_fwd", M, nblocks, p, q, true);
   if (rc) return rc;
+  if (p % 64 != 0 || q % 64 != 0) {               // block sizes off the tile grid (d = 960: 240-wide blocks): the masked kernel
+    hipStream_t st = (hipStream_t)stream;
+    return q >= 128 ? launch_blockdiag<2, 2, true, uint16_t, 2, true>(x, w, nullptr, nullptr, out, M, nblocks, p, q, intermediate, st)
+                    : launch_blockdiag<4, 1, true, uint16_t, 2, true>(x, w, nullptr, nullptr, out, M, nblocks, p, q, intermediate, st);
+  }
   if (q % 128 == 0 && p <= 256) {                 // short K: weight-stationary kernel
     hipStream_t st = (hipStream_t)stream;
     switch (p / 16) {
@@ -994,6 +1015,13 @@ extern "C" int m2_blockdiag_linear_fwd(const void* x, const void* w, const float
   int rc = check_blockdiag("m2_blockdiag_linear_fwd", M, nblocks, p, q, false);
   if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
+  if (p % 64 != 0 || q % 64 != 0) {               // block sizes off the tile grid: the masked kernel
+    if (out_dtype == M2_DTYPE_F32)
+      return q >= 128 ? launch_blockdiag<2, 2, false, float, 1, true>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st)
+                      : launch_blockdiag<4, 1, false, float, 1, true>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st);
+    return q >= 128 ? launch_blockdiag<2, 2, false, uint16_t, 1, true>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st)
+                    : launch_blockdiag<4, 1, false, uint16_t, 1, true>(x, w, bias, residual, out, M, nblocks, p, q, out_features, st);
+  }
   // 256 x 192 tiles once there is at least one per compute unit (measured at d = 768 and 1536: below that the
   // smaller tiles of the general kernel fill the chip better)
   if (q % kWideBN == 0 && (long)((M + kWideBM - 1) / kWideBM) * (nblocks * q / kWideBN) >= num_cus())

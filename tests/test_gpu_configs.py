@@ -67,6 +67,30 @@ def test_config2_full_batch_end_to_end(gpu):
     assert e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
 
 
+@pytest.mark.parametrize("which,L,B", [("m2_bert_110m", 128, 8), ("m2_bert_110m", 2048, 2), ("m2_bert_341m", 128, 4)])
+def test_other_model_widths_every_layer(gpu, which, L, B):
+    """The reference's other two model widths -- 960 (240-wide MLP blocks: off the 64-wide tile grid of the GEMM kernels,
+    bert/yamls/pretrain/monarch-mixer-pretrain-960dim-parameter-matched.yaml) and 1792
+    (monarch-mixer-large-pretrain-1792dim-341m-parameters.yaml) -- every layer within 2e-2 of the fp32 oracle fed the
+    GPU's own previous-layer output, eagerly and as a graph replay."""
+    import m2_amd
+    cfg = getattr(m2_amd, which)(L)
+    cfg.num_hidden_layers = 3
+    sd = m2_amd.seeded_state_dict(cfg, 77)
+    ids = torch.randint(0, cfg.vocab_size, (B, L), generator=torch.Generator().manual_seed(L + B))
+    model = _model(cfg, sd, gpu)
+    errs, layers = _per_layer_errors(model, sd, cfg, ids, gpu, cfg.num_hidden_layers)
+    for i, (e, e2) in enumerate(errs):
+        assert e < TOL_BF16 and e2 < TOL_BF16, (which, i, e, e2)
+    graphed = m2_amd.BertModel(cfg, use_hip_graph=True)
+    graphed.load_state_dict(sd)
+    graphed = graphed.to(gpu).eval()
+    with torch.no_grad():
+        for _ in range(2):
+            out, _ = graphed(ids.to(gpu))
+    assert torch.equal(out.float(), layers[-1].float())
+
+
 def test_config3_every_layer_and_reference_autocast_drift(gpu):
     """(1) Every one of the 12 layers at L = 8192, B = 4 within 2e-2 of the fp32 oracle on the same input.
     (2) End to end, the deviation from the fp32 oracle is compared, layer by layer, with the deviation of the

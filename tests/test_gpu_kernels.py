@@ -176,7 +176,12 @@ def test_plain_fftconv_module_api(gpu):
 
 
 @pytest.mark.parametrize("M,d,I", [(256, 768, 3072), (200, 256, 512), (4096, 1536, 6144), (300, 512, 2048),
-                                   (300, 1024, 4096), (130, 256, 768), (1100, 768, 3072)])
+                                   (300, 1024, 4096), (130, 256, 768), (1100, 768, 3072),
+                                   # block sizes off the 64-wide tile grid: the 960-wide model of the reference
+                                   # (bert/yamls/pretrain/monarch-mixer-pretrain-960dim-parameter-matched.yaml: 240-wide
+                                   # blocks), the 1792-wide one, and small multiples of 8
+                                   (4096, 960, 3840), (333, 960, 3840), (300, 1792, 7168), (200, 32, 64), (130, 96, 352),
+                                   (70, 544, 1120)])
 def test_blockdiag_glu_and_linear(gpu, M, d, I):
     """K3 vs oracle.blockdiag_* on bf16-rounded operands (fp64 reference)."""
     from m2_amd import ops
