@@ -262,6 +262,34 @@ def test_config1_mixer_fp32(gpu):
     assert e < TOL_F32 and e2 < TOL_F32, (e, e2)
 
 
+def test_input_shorter_than_l_max(gpu):
+    """A model built for l_max = 1024 run on 256 positions: the filters are the first 256 rows of the positional
+    embedding and of t, the transform length follows the input (bert/src/mm/hyena_utils.py:201-211,
+    bert/src/mm/monarch_mixer_sequence_mixer.py:104,120-139).  The mixer alone in fp32 at 1e-4, then two encoder layers."""
+    import m2_amd
+    from oracle import m2_oracle as O
+    cfg = m2_amd.m2_bert_80m(1024)
+    cfg.num_hidden_layers = 2
+    sd = m2_amd.seeded_state_dict(cfg, 31, what="mixer")
+    mix = m2_amd.MonarchMixerSequenceMixing(768, l_max=1024, bidirectional=True, hyena_emb_dim=5, hyena_filter_order=128,
+                                            residual_long_conv=True, hyena_w=10, hyena_w_mod=1)
+    mix.load_state_dict(sd)
+    mix = mix.to(gpu).eval()
+    u = torch.randn(3, 256, 768, generator=torch.Generator().manual_seed(8))
+    y, _ = mix(u.to(gpu))
+    e, e2 = rel_err(y, O.mixer_forward(sd, "", u))
+    assert y.shape == u.shape and e < TOL_F32 and e2 < TOL_F32, (e, e2)
+    sd = m2_amd.seeded_state_dict(cfg, 32)
+    model = m2_amd.BertModel(cfg)
+    model.load_state_dict(sd)
+    model = model.to(gpu).eval()
+    ids = torch.randint(0, cfg.vocab_size, (3, 256), generator=torch.Generator().manual_seed(9))
+    mask = torch.ones(3, 256, dtype=torch.long)
+    out, _ = model(ids.to(gpu), attention_mask=mask.to(gpu))
+    e, e2 = rel_err(out, O.model_forward(sd, ids, mask, cfg))
+    assert out.shape == (3, 256, 768) and e < TOL_BF16 and e2 < TOL_BF16, (e, e2)
+
+
 @pytest.mark.parametrize("L,B,layers", [(128, 4, 2), (1024, 2, 2), (16384, 1, 1), (32768, 1, 1)])
 def test_encoder_small(gpu, L, B, layers):
     """Fused encoder schedule and the module-by-module path agree with the oracle (bf16 tolerance)."""
