@@ -1,4 +1,5 @@
-// The gated block-diagonal GEMM with the GELU GLU on its accumulators for 384-wide blocks (d = 1536, nblocks = 4):
+// The gated block-diagonal GEMM with the GELU GLU on its accumulators for 384-wide blocks (d = 1536, nblocks = 4), and,
+// with eight K steps instead of twelve and zeros beyond the block's width, for blocks of 224 .. 248 (d = 960: 240):
 //
 //   h = blockdiag(x, Wg)                      (M, 2I)   never materialised
 //   g = gelu_erf(h[:, :I]) * h[:, I:]         (M, I)    bf16, the input of `wo`
@@ -29,39 +30,50 @@
 
 namespace m2 {
 
-constexpr int kSP = 384;                    // block width of x (d / 4)
-constexpr int kSKS = kSP / 32;              // K steps (K = 32 per MFMA): 12
 constexpr int kSRows = 128;                 // rows per workgroup: 8 waves x 16
 constexpr int kSChunk = 32;                 // gated columns per chunk
 constexpr int kSBlk = 1024;                 // one operand block: 64 lanes x 16 bytes = 16 rows x 32 K
-constexpr int kSStage = 2 * 2 * kSKS * kSBlk;      // (gate | value) x 2 row tiles x 12 K steps = 48 KB
 constexpr int kSStages = 3;
-constexpr int kSLds = kSStages * kSStage;   // 144 KB
-constexpr int kSBatch = 6;                  // direct loads a wave issues per chunk: 48 blocks / 8 waves
+// KS = K steps (K = 32 per MFMA) of a block: 12 for 384-wide blocks, 8 for blocks of up to 256 (the weights and the x
+// rows are zero beyond the block's real width p)
+template <int KS>
+struct GluShape {
+  static constexpr int kStage = 2 * 2 * KS * kSBlk;      // (gate | value) x 2 row tiles x KS K steps: 48 KB / 32 KB
+  static constexpr int kLds = kSStages * kStage;         // 144 KB / 96 KB
+  static constexpr int kBatch = 4 * KS / 8;              // direct loads a wave issues per chunk: blocks / 8 waves
+};
+static int glu_stream_ksteps(int p) { return p == 384 ? 12 : (p >= 224 && p <= 248 && p % 8 == 0) ? 8 : 0; }
 
 // Re-packs gated_layers.weight (4, I / 2, 384) into the image of the LDS stages: for r = 0 .. 3 and chunk c (32 gated
 // columns) 48 blocks of 64 lanes x 16 bytes; block ((value, t), s) = index (2 value + t) 12 + s; lane (i, q) holds row
 // gamma(16 t + i) = 8 (i / 4) + 4 t + i % 4 of the chunk, K = 32 s + 8 q .. + 7.  One thread per 16-byte piece.
-__global__ __launch_bounds__(256) void glu_stream_pack_kernel(const uint16_t* __restrict__ wg, u32x4* __restrict__ packed, int I) {
+template <int KS>
+__global__ __launch_bounds__(256) void glu_stream_pack_kernel(const uint16_t* __restrict__ wg, u32x4* __restrict__ packed, int I, int p) {
+  constexpr int NB = 4 * KS;                 // operand blocks per chunk
   const int IS = I >> 2, q = I >> 1, nchunks = IS / kSChunk;
   const long piece = (long)blockIdx.x * 256 + threadIdx.x;
-  const long npieces = 4l * nchunks * (kSStage / 16);
+  const long npieces = 4l * nchunks * (GluShape<KS>::kStage / 16);
   if (piece >= npieces) return;
   const int lane = piece & 63, i16 = lane & 15, q4 = lane >> 4;
-  const int blk = (piece >> 6) % 48;
-  const int c = (piece / (64 * 48)) % nchunks;
-  const int r = piece / (64l * 48 * nchunks);
-  const int s = blk % kSKS, t = (blk / kSKS) & 1, val = blk / (2 * kSKS);
+  const int blk = (piece >> 6) % NB;
+  const int c = (piece / (64 * NB)) % nchunks;
+  const int r = piece / (64l * NB * nchunks);
+  const int s = blk % KS, t = (blk / KS) & 1, val = blk / (2 * KS);
   const int gamma = 8 * (i16 >> 2) + 4 * t + (i16 & 3);
-  const uint16_t* src = wg + (((long)((r >> 1) + 2 * val) * q + (long)(r & 1) * IS + c * kSChunk + gamma) * kSP + 32 * s + 8 * q4);
-  packed[piece] = *reinterpret_cast<const u32x4*>(src);
+  const int k0 = 32 * s + 8 * q4;
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (k0 < p)
+    v = *reinterpret_cast<const u32x4*>(wg + (((long)((r >> 1) + 2 * val) * q + (long)(r & 1) * IS + c * kSChunk + gamma) * p + k0));
+  packed[piece] = v;
 }
 
+template <int KS>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void glu_stream_kernel(
-    const uint16_t* __restrict__ x,             // (M, 1536) bf16
+    const uint16_t* __restrict__ x,             // (M, 4 p) bf16
     const unsigned char* __restrict__ wpk,      // the gated weight as packed by glu_stream_pack_kernel
     uint16_t* __restrict__ out,                 // (M, I) bf16
-    int M, int I, int ntiles) {
+    int M, int I, int ntiles, int p) {
+  constexpr int kSKS = KS, kSStage = GluShape<KS>::kStage, kSBatch = GluShape<KS>::kBatch;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, i16 = lane & 15, q4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -76,19 +88,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int IS = I >> 2;                  // gated columns of this r
   const int nchunks = IS / kSChunk;
   const int gb = r >> 1;                  // gate block; the value block is gb + 2
-  const int d = 4 * kSP;
+  const int d = 4 * p;
 
   // ---- the wave's x rows as stationary B operands: lane (n, q) holds x[row n][32 s + 8 q .. + 8) of both blocks
   bf16x8 xa[kSKS], xb[kSKS];
   auto load_x = [&](int t) __attribute__((always_inline)) {
     int row = t * kSRows + 16 * wave + i16;
     row = row < M ? row : M - 1;
-    const uint16_t* pa = x + (long)row * d + gb * kSP + 8 * q4;
-    const uint16_t* pb = pa + 2 * kSP;
+    const uint16_t* pa = x + (long)row * d + gb * p + 8 * q4;
+    const uint16_t* pb = pa + 2 * p;
     static_for<0, kSKS>([&](auto ss) {
       constexpr int s = decltype(ss)::value;
-      xa[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pa + 32 * s));
-      xb[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pb + 32 * s));
+      if (KS == 12 || 32 * s + 8 * q4 < p) {      // narrower blocks: zeros beyond the block's width (the weights are zero there too)
+        xa[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pa + 32 * s));
+        xb[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pb + 32 * s));
+      } else {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        xa[s] = __builtin_bit_cast(bf16x8, z);
+        xb[s] = __builtin_bit_cast(bf16x8, z);
+      }
     });
   };
   load_x(tile);
@@ -207,25 +225,46 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 using namespace m2;
 
 extern "C" int m2_glu_stream_supported(int in_features, int intermediate, int nblocks) {
-  return nblocks == 4 && in_features == 4 * kSP && intermediate > 0 && intermediate % (4 * kSChunk) == 0;
+  return nblocks == 4 && in_features > 0 && in_features % 4 == 0 && glu_stream_ksteps(in_features / 4) != 0 && intermediate > 0 &&
+         intermediate % (4 * kSChunk) == 0;
 }
 
 extern "C" long m2_glu_stream_packed_bytes(int in_features, int intermediate, int nblocks) {
   if (!m2_glu_stream_supported(in_features, intermediate, nblocks)) return 0;
-  return 4l * (intermediate / 4 / kSChunk) * kSStage;      // = 2 bytes x elements of w_gated
+  const int ks = glu_stream_ksteps(in_features / 4);
+  return 4l * (intermediate / 4 / kSChunk) * (ks == 12 ? GluShape<12>::kStage : GluShape<8>::kStage);
 }
+
+static const char* kGluStreamShapes =
+    "built for nblocks=4, in_features/4 = 384 or a multiple of 8 in [224, 248], intermediate a multiple of 128";
 
 extern "C" int m2_glu_stream_pack(const void* w_gated, void* packed, int in_features, int intermediate, int nblocks,
                                   void* stream) {
   if (!w_gated || !packed) return set_error(M2_ERR_ARG, "m2_glu_stream_pack: null pointer");
   if (!m2_glu_stream_supported(in_features, intermediate, nblocks))
-    return set_error(M2_ERR_UNSUPPORTED,
-                     "m2_glu_stream_pack: built for nblocks=4, in_features=1536 and intermediate a multiple of 128 "
-                     "(got nblocks=%d in=%d intermediate=%d)", nblocks, in_features, intermediate);
+    return set_error(M2_ERR_UNSUPPORTED, "m2_glu_stream_pack: %s (got nblocks=%d in=%d intermediate=%d)", kGluStreamShapes,
+                     nblocks, in_features, intermediate);
   const long npieces = m2_glu_stream_packed_bytes(in_features, intermediate, nblocks) / 16;
-  hipLaunchKernelGGL(glu_stream_pack_kernel, dim3((unsigned)((npieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const uint16_t*)w_gated, (u32x4*)packed, intermediate);
+  const int p = in_features / 4;
+  const dim3 grid((unsigned)((npieces + 255) / 256));
+  if (glu_stream_ksteps(p) == 12)
+    hipLaunchKernelGGL(glu_stream_pack_kernel<12>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)w_gated,
+                       (u32x4*)packed, intermediate, p);
+  else
+    hipLaunchKernelGGL(glu_stream_pack_kernel<8>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)w_gated,
+                       (u32x4*)packed, intermediate, p);
   return check_launch("glu_stream_pack");
+}
+
+template <int KS>
+static int launch_glu_stream(const void* x, const void* w_packed, void* out, int M, int intermediate, int p, int per_xcd,
+                             int ntiles, hipStream_t stream) {
+  auto kern = glu_stream_kernel<KS>;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, GluShape<KS>::kLds);
+  if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(glu_stream): %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(kern, dim3(8 * per_xcd), dim3(512), GluShape<KS>::kLds, stream, (const uint16_t*)x,
+                     (const unsigned char*)w_packed, (uint16_t*)out, M, intermediate, ntiles, p);
+  return check_launch("glu_stream");
 }
 
 extern "C" int m2_glu_stream_fwd(const void* x, const void* w_packed, void* out, int M, int in_features, int intermediate,
@@ -233,18 +272,14 @@ extern "C" int m2_glu_stream_fwd(const void* x, const void* w_packed, void* out,
   if (!x || !w_packed || !out) return set_error(M2_ERR_ARG, "m2_glu_stream_fwd: null pointer");
   if (M <= 0) return set_error(M2_ERR_ARG, "m2_glu_stream_fwd: M=%d must be positive", M);
   if (!m2_glu_stream_supported(in_features, intermediate, nblocks))
-    return set_error(M2_ERR_UNSUPPORTED,
-                     "m2_glu_stream_fwd: built for nblocks=4, in_features=1536 and intermediate a multiple of 128 "
-                     "(got nblocks=%d in=%d intermediate=%d); use m2_blockdiag_glu_fwd", nblocks, in_features, intermediate);
+    return set_error(M2_ERR_UNSUPPORTED, "m2_glu_stream_fwd: %s (got nblocks=%d in=%d intermediate=%d); use m2_blockdiag_glu_fwd",
+                     kGluStreamShapes, nblocks, in_features, intermediate);
   const int ntiles = (M + kSRows - 1) / kSRows;
-  // one persistent workgroup per compute unit (144 KB of LDS each), an even number per XCD
+  // one persistent workgroup per compute unit (its LDS stages take most of it), an even number per XCD
   int per_xcd = (num_cus() / 8) & ~1;
   if (per_xcd < 2) per_xcd = 2;      // a device (or partition) with fewer than 16 compute units: work is dealt to 8 x per_xcd slots whatever the real count
   if (per_xcd > 2 * ((ntiles + 3) / 4)) per_xcd = 2 * ((ntiles + 3) / 4);
-  auto kern = glu_stream_kernel;
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kSLds);
-  if (e != hipSuccess) return set_error(M2_ERR_LAUNCH, "hipFuncSetAttribute(glu_stream): %s", hipGetErrorString(e));
-  hipLaunchKernelGGL(kern, dim3(8 * per_xcd), dim3(512), kSLds, (hipStream_t)stream, (const uint16_t*)x,
-                     (const unsigned char*)w_packed, (uint16_t*)out, M, intermediate, ntiles);
-  return check_launch("glu_stream");
+  const int p = in_features / 4;
+  return glu_stream_ksteps(p) == 12 ? launch_glu_stream<12>(x, w_packed, out, M, intermediate, p, per_xcd, ntiles, (hipStream_t)stream)
+                                    : launch_glu_stream<8>(x, w_packed, out, M, intermediate, p, per_xcd, ntiles, (hipStream_t)stream);
 }

@@ -339,20 +339,21 @@ def glu_stream_supported(in_features: int, intermediate: int, nblocks: int) -> b
 
 def glu_stream_pack(w_gated: Tensor) -> Tensor:
     """gated_layers.weight (nb, 2I/nb, d/nb) bf16 -> the packed copy `glu_stream` streams (flat bf16 tensor of the
-    weight's size).  Once per set of weights."""
+    weight's size; blocks narrower than 256 are padded to 256 with zeros).  Once per set of weights."""
     nb, q, p = w_gated.shape
     _require(w_gated, "w_gated", torch.bfloat16)
     d, I = nb * p, nb * q // 2
     nbytes = int(lib.m2_glu_stream_packed_bytes(d, I, nb))
     if nbytes == 0:
-        raise RuntimeError(f"glu_stream is built for nblocks=4, in_features=1536, intermediate % 128 == 0; got {nb}, {d}, {I}")
+        raise RuntimeError("glu_stream is built for nblocks=4, blocks 384 wide or a multiple of 8 in [224, 248], "
+                           f"intermediate % 128 == 0; got {nb}, {d}, {I}")
     packed = torch.empty(nbytes // 2, dtype=torch.bfloat16, device=w_gated.device)
     check(lib.m2_glu_stream_pack(_ptr(w_gated), _ptr(packed), d, I, nb, _stream()))
     return packed
 
 
 def glu_stream(x: Tensor, w_gated: Tensor, out: Optional[Tensor] = None, packed: Optional[Tensor] = None) -> Tensor:
-    """gelu_erf(h[:, :I]) * h[:, I:] with h = blockdiag(x, w_gated), as `blockdiag_glu`, for 384-wide blocks.
+    """gelu_erf(h[:, :I]) * h[:, I:] with h = blockdiag(x, w_gated), as `blockdiag_glu`, for 384-wide blocks (d = 1536) and blocks of 224 .. 248 (d = 960).
     x (M, d) bf16, w_gated (nb, 2I/nb, d/nb) bf16; `packed` = glu_stream_pack(w_gated), which a caller with fixed
     weights computes once (without it the weight is packed on every call)."""
     M, d = x.shape

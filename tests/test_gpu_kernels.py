@@ -803,16 +803,19 @@ def test_blockdiag_linear_fp32_outside_autocast(gpu, M, in_f, out_f, nb):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,I", [(1, 6144), (100, 6144), (128, 6144), (300, 1536), (8192, 6144), (8192 - 70, 6144), (130, 256),
-                                 (520, 128)])
-def test_glu_stream_matches_oracle_and_the_tiled_kernel(gpu, M, I):
-    """gated_layers -> GLU for 384-wide blocks (d = 1536) from packed weights, against fp64 on the bf16-rounded
-    operands and against m2_blockdiag_glu_fwd (same arithmetic: bit-close, the accumulation order differs), ragged M,
-    one chunk per r (I = 128), more rows than one round of workgroups."""
+@pytest.mark.parametrize("M,I,d", [(1, 6144, 1536), (100, 6144, 1536), (128, 6144, 1536), (300, 1536, 1536), (8192, 6144, 1536),
+                                   (8192 - 70, 6144, 1536), (130, 256, 1536), (520, 128, 1536),
+                                   (1, 3840, 960), (8192 - 70, 3840, 960), (300, 128, 960), (200, 3840, 896), (200, 1024, 992)])
+def test_glu_stream_matches_oracle_and_the_tiled_kernel(gpu, M, I, d):
+    """gated_layers -> GLU for 384-wide blocks (d = 1536) and for blocks of 224 .. 248 (d = 960: 240 wide, computed as
+    256 with zeros beyond) from packed weights, against fp64 on the bf16-rounded operands and against
+    m2_blockdiag_glu_fwd (same arithmetic: bit-close, the accumulation order differs), ragged M, one chunk per r
+    (I = 128), more rows than one round of workgroups."""
     from m2_amd import ops
     from oracle import m2_oracle as O
-    d, nb = 1536, 4
+    nb = 4
     assert ops.glu_stream_supported(d, I, nb) and not ops.glu_stream_supported(768, 3072, nb)
+    assert not ops.glu_stream_supported(1024, 4096, nb) and not ops.glu_stream_supported(1792, 7168, nb)
     g = torch.Generator().manual_seed(7 * M + I)
     x = torch.randn(M, d, generator=g).bfloat16()
     wg = (torch.randn(nb, 2 * I // nb, d // nb, generator=g) * 0.05).bfloat16()
@@ -827,6 +830,6 @@ def test_glu_stream_matches_oracle_and_the_tiled_kernel(gpu, M, I):
     pk = ops.glu_stream_pack(wg.to(gpu))
     again = ops.glu_stream(x.to(gpu), wg.to(gpu), packed=pk)
     assert torch.equal(again, got)
-    with pytest.raises(RuntimeError, match="1536"):
+    with pytest.raises(RuntimeError, match="384"):
         ops.glu_stream(torch.zeros(8, 768, device=gpu, dtype=torch.bfloat16),
                        torch.zeros(4, 256, 192, device=gpu, dtype=torch.bfloat16))
