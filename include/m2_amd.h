@@ -213,7 +213,7 @@ int m2_mlp_fused_fwd(const void* x, const void* w_packed, const float* bias, con
  * in/nblocks) bf16, gated_layers.weight; packed: m2_glu_stream_packed_bytes bytes of device memory, 16-byte aligned,
  * the size of the weight, or of the weight with its blocks padded to 256 columns when they are narrower).  m2_glu_stream_fwd: x (M, in_features) bf16, w_packed as written by m2_glu_stream_pack for
  * the same shape, out (M, intermediate) bf16.  m2_glu_stream_supported returns 1 for the shapes the kernel is built for
- * (nblocks == 4, in_features / 4 == 384 or a multiple of 8 in [224, 248], intermediate % 128 == 0); for others m2_glu_stream_packed_bytes returns 0, the
+ * (nblocks == 4, in_features / 4 == 384, 448 or a multiple of 8 in [224, 248], intermediate % 128 == 0); for others m2_glu_stream_packed_bytes returns 0, the
  * other two return M2_ERR_UNSUPPORTED and the caller uses m2_blockdiag_glu_fwd. */
 int m2_glu_stream_supported(int in_features, int intermediate, int nblocks);
 long m2_glu_stream_packed_bytes(int in_features, int intermediate, int nblocks);

@@ -33,16 +33,17 @@ namespace m2 {
 constexpr int kSRows = 128;                 // rows per workgroup: 8 waves x 16
 constexpr int kSChunk = 32;                 // gated columns per chunk
 constexpr int kSBlk = 1024;                 // one operand block: 64 lanes x 16 bytes = 16 rows x 32 K
-constexpr int kSStages = 3;
-// KS = K steps (K = 32 per MFMA) of a block: 12 for 384-wide blocks, 8 for blocks of up to 256 (the weights and the x
-// rows are zero beyond the block's real width p)
+// KS = K steps (K = 32 per MFMA) of a block: 12 for 384-wide blocks, 14 for 448-wide ones, 8 for blocks of up to 256
+// (the weights and the x rows are zero beyond the block's real width p).  Three LDS stages (loads two chunks ahead)
+// where they fit, two (one chunk ahead) for the 56 KB chunks of 448-wide blocks.
 template <int KS>
 struct GluShape {
-  static constexpr int kStage = 2 * 2 * KS * kSBlk;      // (gate | value) x 2 row tiles x KS K steps: 48 KB / 32 KB
-  static constexpr int kLds = kSStages * kStage;         // 144 KB / 96 KB
+  static constexpr int kStage = 2 * 2 * KS * kSBlk;      // (gate | value) x 2 row tiles x KS K steps: 32 / 48 / 56 KB
+  static constexpr int kStages = 3 * kStage <= 160 * 1024 ? 3 : 2;
+  static constexpr int kLds = kStages * kStage;          // 96 / 144 / 112 KB
   static constexpr int kBatch = 4 * KS / 8;              // direct loads a wave issues per chunk: blocks / 8 waves
 };
-static int glu_stream_ksteps(int p) { return p == 384 ? 12 : (p >= 224 && p <= 248 && p % 8 == 0) ? 8 : 0; }
+static int glu_stream_ksteps(int p) { return p == 384 ? 12 : p == 448 ? 14 : (p >= 224 && p <= 248 && p % 8 == 0) ? 8 : 0; }
 
 // Re-packs gated_layers.weight (4, I / 2, 384) into the image of the LDS stages: for r = 0 .. 3 and chunk c (32 gated
 // columns) 48 blocks of 64 lanes x 16 bytes; block ((value, t), s) = index (2 value + t) 12 + s; lane (i, q) holds row
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const unsigned char* __restrict__ wpk,      // the gated weight as packed by glu_stream_pack_kernel
     uint16_t* __restrict__ out,                 // (M, I) bf16
     int M, int I, int ntiles, int p) {
-  constexpr int kSKS = KS, kSStage = GluShape<KS>::kStage, kSBatch = GluShape<KS>::kBatch;
+  constexpr int kSKS = KS, kSStage = GluShape<KS>::kStage, kSBatch = GluShape<KS>::kBatch, kSStages = GluShape<KS>::kStages;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, i16 = lane & 15, q4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint16_t* pb = pa + 2 * p;
     static_for<0, kSKS>([&](auto ss) {
       constexpr int s = decltype(ss)::value;
-      if (KS == 12 || 32 * s + 8 * q4 < p) {      // narrower blocks: zeros beyond the block's width (the weights are zero there too)
+      if (KS != 8 || 32 * s + 8 * q4 < p) {      // narrower blocks: zeros beyond the block's width (the weights are zero there too)
         xa[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pa + 32 * s));
         xb[s] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(pb + 32 * s));
       } else {
@@ -133,9 +134,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   };
   u32x4 ring[kPF];
 
-  // prologue: the chunks of iterations 0 and 1
+  // prologue: the chunks of iterations 0 and (three stages) 1
   static_for<0, kSBatch>([&](auto jj) { dma_one(0, 0, jj); });
-  static_for<0, kSBatch>([&](auto jj) { dma_one(1, nchunks > 1 ? 1 : 0, jj); });
+  if constexpr (kSStages == 3) static_for<0, kSBatch>([&](auto jj) { dma_one(1, nchunks > 1 ? 1 : 0, jj); });
   __builtin_amdgcn_s_waitcnt(kWaitVm0);
   __syncthreads();
 
@@ -176,8 +177,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       });
       // the previous chunk leaves while the first operands of this one travel
       if constexpr (!HEAD) finish_chunk(it - 1);
-      const int st2 = st == 0 ? 2 : st - 1;                       // (st + 2) % 3
-      const int c2 = (it + 2) % nchunks;                          // of this tile or, at its end, of the next one
+      const int st2 = st == 0 ? kSStages - 1 : st - 1;            // (st + stages - 1) % stages: the stage read in the iteration before
+      const int c2 = (it + kSStages - 1) % nchunks;               // of this tile or, at its end, of the next one
+      constexpr int kDmaEvery = kSStages == 3 ? 8 : 4;            // one chunk ahead only: the loads go out early in the iteration
       static_for<0, kNM>([&](auto kk) {
         constexpr int k = decltype(kk)::value;
         constexpr int s = k / 4, sel = k % 4, t = sel >> 1, val = sel & 1;
@@ -191,7 +193,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         if constexpr (k + kPF < kNM) ring[k % kPF] = *reinterpret_cast<const u32x4*>(smem + ob + operand_off(ic<k + kPF>{}));
         // the direct loads for iteration n + 2, one every eighth MFMA
-        if constexpr (k % 8 == 1 && k / 8 < kSBatch) dma_one(st2, c2, ic<k / 8>{});
+        if constexpr (k % kDmaEvery == 1 && k / kDmaEvery < kSBatch) dma_one(st2, c2, ic<k / kDmaEvery>{});
         __builtin_amdgcn_sched_barrier(0);
       });
       static_for<0, 8>([&](auto ee) {
@@ -200,10 +202,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         vp[e] = v[e >> 2][e & 3];
       });
       // everything but this wave's newest batch has landed: after the barrier the next chunk is complete for everybody
-      __builtin_amdgcn_s_waitcnt(0x0F70 | kSBatch);
+      if constexpr (kSStages == 3) __builtin_amdgcn_s_waitcnt(0x0F70 | kSBatch);
+      else __builtin_amdgcn_s_waitcnt(kWaitVm0);                  // two stages: the batch just issued is the next chunk
       __syncthreads();
       __builtin_amdgcn_sched_barrier(0);
-      st = st == 2 ? 0 : st + 1;
+      st = st == kSStages - 1 ? 0 : st + 1;
     };
     iteration(ic<1>{}, 0);
     for (int it = 1; it < nchunks; ++it) iteration(ic<0>{}, it);
@@ -232,11 +235,11 @@ extern "C" int m2_glu_stream_supported(int in_features, int intermediate, int nb
 extern "C" long m2_glu_stream_packed_bytes(int in_features, int intermediate, int nblocks) {
   if (!m2_glu_stream_supported(in_features, intermediate, nblocks)) return 0;
   const int ks = glu_stream_ksteps(in_features / 4);
-  return 4l * (intermediate / 4 / kSChunk) * (ks == 12 ? GluShape<12>::kStage : GluShape<8>::kStage);
+  return 4l * (intermediate / 4 / kSChunk) * (ks == 12 ? GluShape<12>::kStage : ks == 14 ? GluShape<14>::kStage : GluShape<8>::kStage);
 }
 
 static const char* kGluStreamShapes =
-    "built for nblocks=4, in_features/4 = 384 or a multiple of 8 in [224, 248], intermediate a multiple of 128";
+    "built for nblocks=4, in_features/4 = 384, 448 or a multiple of 8 in [224, 248], intermediate a multiple of 128";
 
 extern "C" int m2_glu_stream_pack(const void* w_gated, void* packed, int in_features, int intermediate, int nblocks,
                                   void* stream) {
@@ -249,6 +252,9 @@ extern "C" int m2_glu_stream_pack(const void* w_gated, void* packed, int in_feat
   const dim3 grid((unsigned)((npieces + 255) / 256));
   if (glu_stream_ksteps(p) == 12)
     hipLaunchKernelGGL(glu_stream_pack_kernel<12>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)w_gated,
+                       (u32x4*)packed, intermediate, p);
+  else if (glu_stream_ksteps(p) == 14)
+    hipLaunchKernelGGL(glu_stream_pack_kernel<14>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)w_gated,
                        (u32x4*)packed, intermediate, p);
   else
     hipLaunchKernelGGL(glu_stream_pack_kernel<8>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)w_gated,
@@ -280,6 +286,9 @@ extern "C" int m2_glu_stream_fwd(const void* x, const void* w_packed, void* out,
   if (per_xcd < 2) per_xcd = 2;      // a device (or partition) with fewer than 16 compute units: work is dealt to 8 x per_xcd slots whatever the real count
   if (per_xcd > 2 * ((ntiles + 3) / 4)) per_xcd = 2 * ((ntiles + 3) / 4);
   const int p = in_features / 4;
-  return glu_stream_ksteps(p) == 12 ? launch_glu_stream<12>(x, w_packed, out, M, intermediate, p, per_xcd, ntiles, (hipStream_t)stream)
-                                    : launch_glu_stream<8>(x, w_packed, out, M, intermediate, p, per_xcd, ntiles, (hipStream_t)stream);
+  switch (glu_stream_ksteps(p)) {
+    case 12: return launch_glu_stream<12>(x, w_packed, out, M, intermediate, p, per_xcd, ntiles, (hipStream_t)stream);
+    case 14: return launch_glu_stream<14>(x, w_packed, out, M, intermediate, p, per_xcd, ntiles, (hipStream_t)stream);
+    default: return launch_glu_stream<8>(x, w_packed, out, M, intermediate, p, per_xcd, ntiles, (hipStream_t)stream);
+  }
 }

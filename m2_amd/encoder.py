@@ -159,7 +159,7 @@ class BertGatedLinearUnitMLP(nn.Module):
         return ops.blockdiag_linear(g, self.wo.weight_bf16(), self.wo.bias.detach().float().contiguous(), a16,
                                     out_dtype=sum_dtype)
 
-    # True: for 384-wide blocks (d = 1536, four blocks) and 240-wide ones (d = 960) the gated product + GLU runs as the kernel that keeps the x rows
+    # True: for 384-wide blocks (d = 1536, four blocks), 448-wide (d = 1792) and 240-wide ones (d = 960) the gated product + GLU runs as the kernel that keeps the x rows
     # in registers and streams packed weights through LDS (m2_glu_stream_fwd) instead of the LDS-tiled GEMM with a GLU
     # epilogue (m2_blockdiag_glu_fwd).  Same arithmetic; other shapes take the tiled kernel.
     stream_glu = True

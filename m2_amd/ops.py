@@ -345,7 +345,7 @@ def glu_stream_pack(w_gated: Tensor) -> Tensor:
     d, I = nb * p, nb * q // 2
     nbytes = int(lib.m2_glu_stream_packed_bytes(d, I, nb))
     if nbytes == 0:
-        raise RuntimeError("glu_stream is built for nblocks=4, blocks 384 wide or a multiple of 8 in [224, 248], "
+        raise RuntimeError("glu_stream is built for nblocks=4, blocks 384 or 448 wide or a multiple of 8 in [224, 248], "
                            f"intermediate % 128 == 0; got {nb}, {d}, {I}")
     packed = torch.empty(nbytes // 2, dtype=torch.bfloat16, device=w_gated.device)
     check(lib.m2_glu_stream_pack(_ptr(w_gated), _ptr(packed), d, I, nb, _stream()))
@@ -353,7 +353,7 @@ def glu_stream_pack(w_gated: Tensor) -> Tensor:
 
 
 def glu_stream(x: Tensor, w_gated: Tensor, out: Optional[Tensor] = None, packed: Optional[Tensor] = None) -> Tensor:
-    """gelu_erf(h[:, :I]) * h[:, I:] with h = blockdiag(x, w_gated), as `blockdiag_glu`, for 384-wide blocks (d = 1536) and blocks of 224 .. 248 (d = 960).
+    """gelu_erf(h[:, :I]) * h[:, I:] with h = blockdiag(x, w_gated), as `blockdiag_glu`, for 384-wide blocks (d = 1536), 448-wide ones (d = 1792) and blocks of 224 .. 248 (d = 960).
     x (M, d) bf16, w_gated (nb, 2I/nb, d/nb) bf16; `packed` = glu_stream_pack(w_gated), which a caller with fixed
     weights computes once (without it the weight is packed on every call)."""
     M, d = x.shape

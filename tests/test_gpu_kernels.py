@@ -805,17 +805,18 @@ def test_blockdiag_linear_fp32_outside_autocast(gpu, M, in_f, out_f, nb):
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,I,d", [(1, 6144, 1536), (100, 6144, 1536), (128, 6144, 1536), (300, 1536, 1536), (8192, 6144, 1536),
                                    (8192 - 70, 6144, 1536), (130, 256, 1536), (520, 128, 1536),
-                                   (1, 3840, 960), (8192 - 70, 3840, 960), (300, 128, 960), (200, 3840, 896), (200, 1024, 992)])
+                                   (1, 3840, 960), (8192 - 70, 3840, 960), (300, 128, 960), (200, 3840, 896), (200, 1024, 992),
+                                   (1, 7168, 1792), (8192 - 70, 7168, 1792), (300, 128, 1792), (33000, 256, 1792)])
 def test_glu_stream_matches_oracle_and_the_tiled_kernel(gpu, M, I, d):
-    """gated_layers -> GLU for 384-wide blocks (d = 1536) and for blocks of 224 .. 248 (d = 960: 240 wide, computed as
-    256 with zeros beyond) from packed weights, against fp64 on the bf16-rounded operands and against
+    """gated_layers -> GLU for 384-wide blocks (d = 1536), 448-wide ones (d = 1792: two LDS stages instead of three) and
+    blocks of 224 .. 248 (d = 960: 240 wide, computed as 256 with zeros beyond) from packed weights, against fp64 on the bf16-rounded operands and against
     m2_blockdiag_glu_fwd (same arithmetic: bit-close, the accumulation order differs), ragged M, one chunk per r
     (I = 128), more rows than one round of workgroups."""
     from m2_amd import ops
     from oracle import m2_oracle as O
     nb = 4
     assert ops.glu_stream_supported(d, I, nb) and not ops.glu_stream_supported(768, 3072, nb)
-    assert not ops.glu_stream_supported(1024, 4096, nb) and not ops.glu_stream_supported(1792, 7168, nb)
+    assert not ops.glu_stream_supported(1024, 4096, nb) and not ops.glu_stream_supported(2048, 8192, nb)
     g = torch.Generator().manual_seed(7 * M + I)
     x = torch.randn(M, d, generator=g).bfloat16()
     wg = (torch.randn(nb, 2 * I // nb, d // nb, generator=g) * 0.05).bfloat16()
