@@ -834,3 +834,4 @@ def test_glu_stream_matches_oracle_and_the_tiled_kernel(gpu, M, I, d):
     with pytest.raises(RuntimeError, match="384"):
         ops.glu_stream(torch.zeros(8, 768, device=gpu, dtype=torch.bfloat16),
                        torch.zeros(4, 256, 192, device=gpu, dtype=torch.bfloat16))
+
