@@ -54,6 +54,39 @@ def test_hyena_filter_taps(gpu, L, std):
         assert rel_err(hr.cpu(), kr.T[None])[0] < max(2e-5, 4 * e32)
 
 
+@pytest.mark.parametrize("L,emb_dim,w,w_mod,shift", [(256, 3, 4, 2, 0.05), (256, 7, 14, 1, 0.0), (2048, 3, 10, 2, 0.05),
+                                                     (2048, 7, 1, 1, -0.02)])
+def test_hyena_filter_settings_off_the_default(gpu, L, emb_dim, w, w_mod, shift):
+    """The filter with the other settings its constructor takes (bert/src/mm/hyena_utils.py:115-166): emb_dim 3 and 7
+    (one and three frequency bands), the Sin frequency w, the multiplier w_mod and a modulation shift -- taps of
+    HyenaFilter.filter / filter_rev against the fp64 oracle (fp32 yardstick as above), and the spectra of the batched
+    call (one-kernel route at L = 256, fused hidden + projection at L = 2048) against the two-step route."""
+    import m2_amd
+    from m2_amd import ops
+    from oracle import m2_oracle as O
+    d = 192
+    torch.manual_seed(L + emb_dim)
+    fn = m2_amd.HyenaFilter(d, emb_dim=emb_dim, order=128, seq_len=L, bidirectional=True, w=w, w_mod=w_mod, shift=shift)
+    with torch.no_grad():
+        for prm in fn.parameters():
+            if prm.dim() == 2:
+                prm.normal_(0.0, 0.05)
+    fn = fn.to(gpu)
+    sd = {"f." + k: v.detach().cpu() for k, v in fn.state_dict().items()}
+    sd64 = O.cast_state_dict(sd, torch.float64)
+    taps = fn.bidirectional_taps(L)
+    for rev, got in ((False, fn.filter(L)), (True, fn.filter_rev(L))):
+        ref = O.hyena_filter_taps(sd64, "f.", L, rev=rev, w_mod=w_mod, shift=shift)
+        e32 = rel_err(O.hyena_filter_taps(sd, "f.", L, rev=rev, w_mod=w_mod, shift=shift), ref)[0]
+        assert rel_err(got.cpu(), ref)[0] < max(2e-5, 4 * e32), (rev, e32)
+    params = fn.kernel_params("both")
+    skip = fn.bias.detach().float().contiguous()
+    table = ops.FilterTable([[params]], [[skip]], L, d, 128, emb_dim)
+    spec = ops.mixer_filter_spectra(table, w_mod=float(w_mod), shift=float(shift))[0]
+    two_step = ops.filter_spectrum(taps, None, skip, None)
+    assert rel_err(spec, two_step)[0] < TOL_F32
+
+
 @pytest.mark.parametrize("L", [128, 256, 512, 1024, 2048])
 @pytest.mark.parametrize("bidirectional,residual", [(True, True), (False, True), (True, False)])
 def test_mixer_filter_spectra_batched(gpu, L, bidirectional, residual):
