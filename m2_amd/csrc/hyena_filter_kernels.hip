@@ -15,7 +15,9 @@
 // (h3 = hi + lo to 16 mantissa bits).  `project_kernel` is the 128 -> d projection as a three-product split-bf16
 // MFMA GEMM (W_hi h_hi + W_hi h_lo + W_lo h_hi, fp32 accumulate; 4.6e-6 relative error against fp64, measured)
 // whose epilogue applies the decay and stores the taps channel-major, forward taps at [0, L) and reverse taps
-// mirrored into [L, 2L).
+// mirrored into [L, 2L).  For L >= 1024 the last two are one launch (`hidden_kernel<2, ., PROJECT = true>`: the
+// workgroup that evaluated the hidden layers of 64 positions goes on to project them, h3 never leaves LDS); for
+// L <= 512 the batched entry point hands h3 to the projection + spectrum kernel of filter_fused_kernels.hip instead.
 #include <hip/hip_runtime.h>
 
 #include <mutex>
