@@ -49,7 +49,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # rocprofv3) but by the two --pmc runs summarised in profiles/encoder_fwd_L8192_B4_hbm_traffic.md (FETCH_SIZE scaled
 # by 2.000, WRITE_SIZE by 1.000 against a plain 256 MiB copy).  Stamped with the state of the kernel it was taken
 # from; reported only for --config c3, with the stamp beside it.
-MIXER_CORE_TRAFFIC_C3 = {"bytes": int((191421 * 2.0 + 55749 * 1.0) * 1024), "kernel": "mixer_split_kernel",
+MIXER_CORE_TRAFFIC_C3 = {"bytes": int((191523 * 2.0 + 55798 * 1.0) * 1024), "kernel": "mixer_split_kernel",
                          "measured": "2026-11-25", "commit": "3e876ed",
                          "source": "profiles/encoder_fwd_L8192_B4_hbm_traffic.md"}
 
