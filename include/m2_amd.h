@@ -103,7 +103,8 @@ int m2_hyena_filter_fwd_static(const m2_hyena_filter_params* params, int nfilter
  * skip_dev    DEVICE array of nmixers * filters_per_mixer pointers to the (d) fp32 skip weights (filter_fn.bias),
  *             entries may be null; the array itself may be NULL (no skip weights).
  * workspace   m2_mixer_filters_workspace_bytes(...) bytes of device memory, 256-byte aligned.
- * spec        nmixers consecutive buffers of m2_filter_spectrum_bytes(d, L) bytes. */
+ * spec        nmixers consecutive buffers of m2_filter_spectrum_bytes(d, L) bytes.
+ * At most 65535 MLPs per call (two per filter): nmixers * filters_per_mixer * 2 <= 65535. */
 size_t m2_mixer_filters_workspace_bytes(int nmixers, int filters_per_mixer, int L, int d, int order);
 int m2_mixer_filters_fwd(const m2_hyena_filter_params* params_dev, const float* const* skip_dev, int nmixers,
                          int filters_per_mixer, int L, int d, int order, int emb_dim, float w_mod, float shift,

@@ -637,9 +637,12 @@ extern "C" int m2_mixer_filters_fwd(const m2_hyena_filter_params* params_dev, co
                                     float shift, void* workspace, float* spec, void* stream) {
   const char* who = "m2_mixer_filters_fwd";
   if (!params_dev || !workspace || !spec) return set_error(M2_ERR_ARG, "%s: null pointer", who);
-  if (nmixers < 1 || nmixers > 16384) return set_error(M2_ERR_ARG, "%s: nmixers=%d not in [1, 16384]", who, nmixers);
   if (filters_per_mixer < 1 || filters_per_mixer > 2)
     return set_error(M2_ERR_ARG, "%s: filters_per_mixer=%d must be 1 or 2", who, filters_per_mixer);
+  // the MLPs of the batch (two per filter) are one grid dimension of the hidden-layer launch
+  if (nmixers < 1 || (long)nmixers * filters_per_mixer * 2 > 65535)
+    return set_error(M2_ERR_ARG, "%s: nmixers=%d with %d filters each: at most 65535 MLPs (two per filter) per call", who, nmixers,
+                     filters_per_mixer);
   int rc = check_filter_sizes(who, L, d, order, emb_dim);
   if (rc) return rc;
   if (!m2_fftconv_supported_seqlen(L))

@@ -54,6 +54,10 @@ def test_size_queries_and_argument_checks_without_gpu():
     assert lib.m2_blockdiag_glu_fwd(one, one, one, 8, 768, 3072, 3, None) == -2
     assert lib.m2_blockdiag_linear_fwd(one, one, None, None, one, 8, 100, 64, 4, 1, None) == -2
     assert lib.m2_layernorm_fwd(one, one, one, 1e-12, None, None, None, 4, 100, None) == -2
+    # the MLPs of a batch of mixers are one grid dimension: 16384 mixers with two filters each would be 65536 of them
+    assert lib.m2_mixer_filters_fwd(one, None, 16384, 2, 128, 768, 128, 5, 1.0, 0.0, one, one, None) == -1
+    assert b"65535" in lib.m2_last_error()
+    assert lib.m2_mixer_filters_fwd(one, None, 4, 3, 128, 768, 128, 5, 1.0, 0.0, one, one, None) == -1
     with pytest.raises(RuntimeError):
         _lib.check(-2)
 
