@@ -431,6 +431,7 @@ extern "C" int m2_mixer_core_fwd(const void* xproj, const float* proj_bias, cons
                                  void* stream) {
   if (!xproj || !short_w || !short_b || !spec || !y) return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: null pointer");
   if (B <= 0 || d <= 0 || d % 8 != 0) return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: need B > 0 and d a positive multiple of 8 (B=%d d=%d)", B, d);
+  if ((long)B * 3 * d > 0x7fffffffL) return set_error(M2_ERR_UNSUPPORTED, "m2_mixer_core_fwd: B * 3 d = %ld rows do not fit an int", (long)B * 3 * d);
   if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
     return set_error(M2_ERR_ARG, "m2_mixer_core_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
   if (!m2_fftconv_supported_seqlen(L))
@@ -455,6 +456,7 @@ extern "C" int m2_fftconv_fwd(const void* x, const float* spec, void* y, int B, 
                               void* stream) {
   if (!x || !spec || !y) return set_error(M2_ERR_ARG, "m2_fftconv_fwd: null pointer");
   if (B <= 0 || d <= 0 || d % 8 != 0) return set_error(M2_ERR_ARG, "m2_fftconv_fwd: need B > 0 and d a positive multiple of 8 (B=%d d=%d)", B, d);
+  if ((long)B * d > 0x7fffffffL) return set_error(M2_ERR_UNSUPPORTED, "m2_fftconv_fwd: B * d = %ld rows do not fit an int", (long)B * d);
   if (act_dtype != M2_DTYPE_F32 && act_dtype != M2_DTYPE_BF16)
     return set_error(M2_ERR_ARG, "m2_fftconv_fwd: act_dtype %d is neither M2_DTYPE_F32 nor M2_DTYPE_BF16", act_dtype);
   if (!m2_fftconv_supported_seqlen(L))
