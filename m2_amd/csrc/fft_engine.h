@@ -289,10 +289,11 @@ __device__ __forceinline__ void forward_to_pairs(cf (&x)[16], int t, float2* row
   dif<8, 8, 16>(x);
 }
 
-// One spectral pair: za sits at frequency k, zb at N-k.  Returns W[k] in za and W[N-k] in zb.
+// One spectral pair: za sits at frequency k, zb at N-k.  Returns W[k] in za and W[N-k] in zb.  The 1/2 of the even/odd
+// separation is folded into the stored spectra (store_filter_spectrum).
 __device__ __forceinline__ void pair_multiply(cf& za, cf& zb, float4 K) {
-  cf A = {0.5f * (za.re + zb.re), 0.5f * (za.im - zb.im)};        // (Z[k] + conj Z[N-k]) / 2
-  cf Bq = {0.5f * (za.im + zb.im), 0.5f * (zb.re - za.re)};       // (Z[k] - conj Z[N-k]) / (2i)
+  cf A = {za.re + zb.re, za.im - zb.im};                          // Z[k] + conj Z[N-k]
+  cf Bq = {za.im + zb.im, zb.re - za.re};                         // (Z[k] - conj Z[N-k]) / i
   cf Pp = cmul(A, cf{K.x, K.y});
   cf Q = cmul(Bq, cf{K.z, K.w});
   za = {Pp.re - Q.im, Pp.im + Q.re};                               // P + iQ
@@ -331,8 +332,8 @@ __device__ __forceinline__ void inverse_from_pairs(cf (&x)[16], int t, float2* r
 // After forward_to_pairs on z = k1 + i k2 (two real filters packed into one complex row): separates the two
 // spectra and stores them in the order the mixer core's multiply reads them, sp[slot * T] as float4 = (K1.re,
 // K1.im, K2.re, K2.im) for the frequency in slot `slot` of this work item's group; work item 0 holds DC and Nyquist
-// (real, packed into slot 0) and the two self-mirrored groups.  `scale` carries the 1/2 of the separation and the
-// 1/N of the convolution.
+// (real, packed into slot 0: multiplied directly, so without the two halves) and the two self-mirrored groups.
+// `scale` carries the 1/2 of this separation, the 1/2 of the separation in pair_multiply and the 1/N of the convolution.
 template <class P>
 __device__ __forceinline__ void store_filter_spectrum(const cf (&x)[16], int t, float scale, float4* __restrict__ sp) {
   float4 K[8];
@@ -348,7 +349,7 @@ __device__ __forceinline__ void store_filter_spectrum(const cf (&x)[16], int t, 
     });
   } else {
     const cf z0 = x[bitrev(0, 3)], z4 = x[bitrev(4, 3)];
-    K[0] = make_float4(2.f * scale * z0.re, 2.f * scale * z4.re, 2.f * scale * z0.im, 2.f * scale * z4.im);
+    K[0] = make_float4(4.f * scale * z0.re, 4.f * scale * z4.re, 4.f * scale * z0.im, 4.f * scale * z4.im);
     static_for<1, 4>([&](auto jj) {
       constexpr int j = decltype(jj)::value;
       K[j] = split(x[bitrev(j, 3)], x[bitrev(8 - j, 3)]);

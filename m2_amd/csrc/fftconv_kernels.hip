@@ -278,7 +278,7 @@ __global__ __launch_bounds__(P::WG) void filter_spectrum_kernel(
   twiddles_init<P>(tw, t, lds + P::RPW * P::ROW_LDS);
   int g, g2;
   paired_groups<P>(t, g, g2);
-  const float scale = 0.5f / (float)N;       // the 1/2 of the even/odd split and the 1/N of the convolution
+  const float scale = 0.25f / (float)N;      // the 1/2 of the even/odd split here, the 1/2 of the one in the mixer core's multiply, the 1/N of the convolution
 
   for (int r0 = blockIdx.x * P::RPW; r0 < d; r0 += gridDim.x * P::RPW) {
     const int r = r0 + rloc;

@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kFusedRows* P::T) void project_spectrum_kernel(
   cf x[16];
   fwd_load<P, P::R1, P::S1>(x, t, row);
   forward_to_pairs<P, false>(x, t, row, tw, g, g2);
-  const float scale = 0.5f / (float)N;       // the 1/2 of the even/odd split and the 1/N of the convolution
+  const float scale = 0.25f / (float)N;      // the 1/2 of the even/odd split here, the 1/2 of the one in the mixer core's multiply, the 1/N of the convolution
   store_filter_spectrum<P>(x, t, scale, spec + (long)mixer * spec_stride4 + (long)c * 8 * T + t);
 }
 
